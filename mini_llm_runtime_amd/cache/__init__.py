@@ -2,10 +2,11 @@
 
 from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
 from .manager import CacheManager, CacheStats, KVGroup, RequestCache, StepLayout, VisibilityError
-from .spec import PagedKVSpec, PagedSpec, SiteCacheSpec, SlotSpec, SlotStateSpec
+from .spec import CompositeSpec, PagedKVSpec, PagedSpec, SiteCacheSpec, SlotSpec, SlotStateSpec
 from .views import KVView, StateView
 
 __all__ = [
+    "CompositeSpec",
     "BlockAllocator",
     "BlockPoolExhaustedError",
     "CacheManager",

@@ -29,7 +29,7 @@ import numpy as np
 import torch
 
 from .block_pool import BlockAllocator, BlockPoolExhaustedError, SlotPool, blocks_for
-from .spec import PagedSpec, SiteCacheSpec, SlotSpec
+from .spec import CompositeSpec, PagedSpec, SiteCacheSpec, SlotSpec
 
 SiteSpec = Optional[SiteCacheSpec]
 
@@ -76,14 +76,25 @@ class KVGroup:
     def num_blocks(self) -> int:
         return self.allocator.total_blocks
 
+    @property
+    def stride(self) -> int:
+        """Tokens per cached entry (1: an entry per token)."""
+        return int(getattr(self.spec, "tokens_per_entry", 1))
+
+    def blocks_for_tokens(self, num_tokens: int) -> int:
+        """Pages that hold the entries of a request of `num_tokens` tokens."""
+        return blocks_for(self.spec.entries_for(num_tokens), self.block_size)
+
     def dead_blocks(self, num_tokens: int) -> int:
         """How many leading pages no query at position >= num_tokens can see."""
+        if self.stride != 1:
+            return 0  # entries of several tokens stay
         return max(0, self.spec.first_live_position(num_tokens) // self.block_size)
 
     def lifetime_blocks(self, max_tokens: int, max_step_tokens: int) -> int:
         """Most pages a request holds at one time over its life."""
-        full = blocks_for(max_tokens, self.block_size)
-        span = self.spec.live_span()
+        full = self.blocks_for_tokens(max_tokens)
+        span = self.spec.live_span() if self.stride == 1 else None
         if span is None:
             return full
         # what the first query of a step may still see (a window, the run of a chunked mask), the
@@ -233,8 +244,9 @@ class CacheManager:
         self.site_specs = tuple(site_specs)
 
         # every spec attaches its site to one of the two stores
-        self._paged_sites: dict[PagedSpec, list[int]] = {}
-        self.state_banks: dict[int, StateBank] = {}
+        # a site is named by its index, a member of a site's composite spec by (index, member name)
+        self._paged_sites: dict[PagedSpec, list] = {}
+        self.state_banks: dict = {}
         for site, spec in enumerate(self.site_specs):
             if spec is not None:
                 spec.attach(self, site)
@@ -246,7 +258,7 @@ class CacheManager:
             KVGroup(i, spec, sites, int(counts[i]), self.block_size, dtype, self.device)
             for i, (spec, sites) in enumerate(grouped.items())
         ]
-        self._site_group: dict[int, KVGroup] = {s: g for g in self.groups for s in g.sites}
+        self._site_group: dict = {s: g for g in self.groups for s in g.sites}
         self.slots = SlotPool(self.max_requests)
         self._requests: dict[str, RequestCache] = {}
         self._pending: Optional[list[_PendingEntry]] = None
@@ -273,13 +285,25 @@ class CacheManager:
             raise KeyError(f"unknown request {request_id!r}") from None
 
     # ---- what the specs call -------------------------------------------------------------------
-    def add_paged_site(self, site: int, spec: PagedSpec) -> None:
+    def add_paged_site(self, site, spec: PagedSpec) -> None:
         """`site` keeps something per token in pages; sites with equal specs share a pool."""
         self._paged_sites.setdefault(spec, []).append(site)
 
-    def add_slot_site(self, site: int, spec: SlotSpec) -> None:
+    def add_slot_site(self, site, spec: SlotSpec) -> None:
         """`site` keeps a state of fixed size per request."""
         self.state_banks[site] = StateBank(site, spec, self.max_requests, self.device)
+
+    def _spec_at(self, key) -> SiteSpec:
+        """The spec that lives under a site index or under a path (site, member name, ...)."""
+        path = key if isinstance(key, tuple) else (key,)
+        if not (isinstance(path[0], (int, np.integer)) and 0 <= path[0] < len(self.site_specs)):
+            return None
+        spec = self.site_specs[path[0]]
+        for name in path[1:]:
+            if not isinstance(spec, CompositeSpec) or name not in spec.members:
+                return None
+            spec = spec.members[name]
+        return spec
 
     def group_of_site(self, site: int) -> KVGroup:
         return self._site_group[site]
@@ -294,7 +318,15 @@ class CacheManager:
         """What the mixer at execution site `site` is handed of the cache that site `owner` keeps
         (its own, or an earlier site's that it only reads), for a step whose metadata is given per
         pool (block tables, slot mappings) and per entry (state rows); None when `owner` keeps nothing.
-        The view is made by the owner's spec."""
+        The view is made by the owner's spec; a composite spec's members make one each, handed over
+        as a dictionary by member name."""
+        spec = self._spec_at(owner)
+        if isinstance(spec, CompositeSpec):
+            path = owner if isinstance(owner, tuple) else (owner,)
+            return {
+                name: self.site_view(site, (*path, name), block_tables, slot_mappings, state_read, state_write)
+                for name in spec.members
+            }
         group = self._site_group.get(owner)
         if group is not None:
             return group.spec.view(
@@ -302,7 +334,7 @@ class CacheManager:
                 block_table=block_tables[group.index],
                 slot_mapping=slot_mappings[group.index],
                 block_size=self.block_size,
-                writable=site == owner,
+                writable=site == (owner[0] if isinstance(owner, tuple) else owner),
                 site=site,
                 owner=owner,
                 tracker=self.visibility_tracker,
@@ -327,14 +359,14 @@ class CacheManager:
         """What a `KVView` reports to: this manager when the check is on, else None."""
         return self if self.check_visibility else None
 
-    def note_write(self, site: int, owner: int) -> None:
+    def note_write(self, site: int, owner) -> None:
         if self._pending is None:
             raise VisibilityError(f"site {site} wrote keys and values outside a step")
-        if site != owner:
+        if site != (owner[0] if isinstance(owner, tuple) else owner):
             raise VisibilityError(f"site {site} wrote into the pages of site {owner}, which it only reads")
         self._written_sites.add(owner)
 
-    def note_read(self, site: int, owner: int) -> None:
+    def note_read(self, site: int, owner) -> None:
         if self._pending is None:
             raise VisibilityError(f"site {site} read the cache outside a step")
         if owner not in self._written_sites:
@@ -434,7 +466,7 @@ class CacheManager:
                 pending.append(entry)
                 for i, g in enumerate(self.groups):
                     have = len(request.tables[i])
-                    need = blocks_for(request.num_tokens + int(n), self.block_size) - have
+                    need = g.blocks_for_tokens(request.num_tokens + int(n)) - have
                     if need <= 0:
                         continue
                     promised = min(need, request.reserved[i])
@@ -521,21 +553,32 @@ class CacheManager:
                 a, b = int(cu_q[r]), int(cu_q[r + 1])
                 positions[a:b] = np.arange(q_starts[r], context[r], dtype=np.int32)
                 token_entry[a:b] = r
-        used = (context + (bs - 1)) // bs  # pages each entry has with this step's tokens
-        width = max(1, int(used.max()))
+        width = max(1, int(((context + (bs - 1)) // bs).max()))  # every pool's table is this wide
         block_tables: list[np.ndarray] = []
         slot_mappings: list[np.ndarray] = []
         for i, g in enumerate(self.groups):
+            stride = g.stride
+            held = context // stride  # entries each request has with this step's tokens
+            used = (held + (bs - 1)) // bs
             table = np.full((count, width), -1, dtype=np.int32)
             for r, e in enumerate(pending):
                 n = int(used[r])
                 table[r, :n] = e.request.table_array(i)[:n]
-            pages = table[token_entry, positions // bs]
+            if stride == 1:
+                index, writes = positions, None
+            else:  # only a token that completes a run of `stride` positions has an entry to write
+                index, writes = positions // stride, (positions + 1) % stride == 0
+            pages = table[token_entry, np.minimum(index // bs, width - 1)]
+            if writes is not None:
+                pages = np.where(writes, pages, 0)
             if (pages < 0).any():
                 r = int(token_entry[int(np.argmax(pages < 0))])
                 raise RuntimeError(f"request {pending[r].request.request_id!r}: a new token has no page")
+            slots = (pages * bs + index % bs).astype(np.int32)
+            if writes is not None:
+                slots = np.where(writes, slots, -1).astype(np.int32)
             block_tables.append(table)
-            slot_mappings.append((pages * bs + positions % bs).astype(np.int32))
+            slot_mappings.append(slots)
         slot_ids = np.array([e.request.slot for e in pending], dtype=np.int32)
         parity = np.array([e.request.state_parity for e in pending], dtype=np.int32)
         return StepLayout(
@@ -563,8 +606,10 @@ class CacheManager:
             for request in self._requests.values():
                 live = len(request.live_blocks(i))
                 dead_tokens = (len(request.tables[i]) - live) * self.block_size
-                committed += max(0, request.num_tokens - dead_tokens)
-                pending += request.pending_tokens
+                committed += max(0, g.spec.entries_for(request.num_tokens) - dead_tokens)
+                pending += g.spec.entries_for(request.num_tokens + request.pending_tokens) - g.spec.entries_for(
+                    request.num_tokens
+                )
             allocated = held * self.block_size
             out.append(
                 CacheStats(

@@ -12,7 +12,7 @@ step function asks what class a spec is.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Optional
+from typing import Any, Mapping, Optional
 
 import torch
 
@@ -44,10 +44,21 @@ class PagedSpec(SiteCacheSpec):
     chunk: an integer C likewise keeps only the run of C positions (runs counted from position 0)
     that the next query lies in: a query never sees beyond the start of its own run.
     The manager asks `first_live_position` and `live_span`, never which of the two it is.
+
+    tokens_per_entry: 1 keeps something for every token.  An integer P > 1 keeps ONE entry for every
+    run of P positions (runs counted from position 0), made when the run's last token comes in: the
+    pool's pages then hold `block_size` entries each, a request of n tokens owns floor(n / P) entries,
+    and the slot mapping of a step names a slot only for the tokens that complete a run (-1 for the
+    others).  Windows and chunks are counted in tokens and do not go with it.
     """
 
     window: Optional[int] = None
     chunk: Optional[int] = None
+    tokens_per_entry: int = 1
+
+    def entries_for(self, num_tokens: int) -> int:
+        """Entries that a request of `num_tokens` tokens owns."""
+        return num_tokens // self.tokens_per_entry
 
     def first_live_position(self, num_tokens: int) -> int:
         """The first position that a query at position >= num_tokens may still see."""
@@ -87,6 +98,39 @@ class PagedSpec(SiteCacheSpec):
         raise NotImplementedError
 
 
+class CompositeSpec(SiteCacheSpec):
+    """Several caches of one site, each under a name: pages of one kind beside pages of another,
+    beside fixed-size states.  Every member attaches itself to its own store under the path (site,
+    name); a member may be a composite again, whose members then live under (site, name, name).  The
+    site's parts are handed a dictionary name -> view (nested likewise).  Two composites are equal
+    when their members are."""
+
+    def __init__(self, members: Mapping[str, SiteCacheSpec]) -> None:
+        if not members:
+            raise ValueError("a composite cache spec needs at least one member")
+        for name, member in members.items():
+            if not isinstance(name, str) or not name or not isinstance(member, SiteCacheSpec):
+                raise ValueError("members of a composite cache spec are specs under non-empty names")
+        self.members: dict[str, SiteCacheSpec] = dict(members)
+
+    def __eq__(self, other: Any) -> bool:
+        return isinstance(other, CompositeSpec) and self.members == other.members
+
+    def __hash__(self) -> int:
+        return hash(tuple(self.members.items()))
+
+    def __repr__(self) -> str:
+        return f"CompositeSpec({self.members!r})"
+
+    def attach(self, manager: Any, site: Any) -> None:
+        path = site if isinstance(site, tuple) else (site,)
+        for name, member in self.members.items():
+            member.attach(manager, (*path, name))
+
+    def page_bytes(self, block_size: int, element_size: int) -> int:
+        return sum(member.page_bytes(block_size, element_size) for member in self.members.values())
+
+
 class SlotSpec(SiteCacheSpec):
     """State of fixed size per request."""
 
@@ -121,10 +165,13 @@ class PagedKVSpec(PagedSpec):
     window: Optional[int] = None
     value_head_dim: Optional[int] = None
     chunk: Optional[int] = None
+    tokens_per_entry: int = 1
 
     def __post_init__(self) -> None:
         if self.num_kv_heads <= 0 or self.head_dim <= 0:
             raise ValueError("PagedKVSpec sizes must be > 0")
+        if self.tokens_per_entry <= 0 or (self.tokens_per_entry > 1 and (self.window or self.chunk)):
+            raise ValueError("PagedKVSpec.tokens_per_entry must be > 0, and 1 under a window or a chunked mask")
         if self.window is not None and self.window <= 0:
             raise ValueError("PagedKVSpec.window must be > 0 or None")
         if self.chunk is not None and (self.chunk <= 0 or self.window is not None):

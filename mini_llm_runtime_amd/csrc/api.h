@@ -157,12 +157,17 @@ int mlr_gemm_merge_fused_bf16(const float* attn_partial, const int* context_lens
 // pages are laid out as for mlr_rope_kv_write.
 // A page id outside [0, num_pages) among the visible keys gives a NaN row.
 // sinks (float32 [heads], or null): the softmax's denominator also holds exp(sinks[head]).
+// pool > 0 (with a window): beside its window a query also sees pooled entries, one key and value for every
+// run of `pool` positions whose last position is <= p - window, read from pages of their own (same layout,
+// `block_size` entries a page, entry b of a request at pooled_table[entry][b / block_size]) in the same softmax.
 int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_pages,
                                const void* value_pages, const int* block_table, int table_width,
                                const int* token_entry, const int* positions, void* out, int dtype,
                                int tokens, int entries, int heads, int kv_heads, int head_dim,
                                int block_size, int num_pages, float scale, int window, int chunk,
-                               const float* sinks, hipStream_t stream);
+                               const float* sinks, const void* pooled_keys, const void* pooled_values,
+                               const int* pooled_table, int pooled_width, int pooled_pages, int pool,
+                               hipStream_t stream);
 
 // x (float32 [rows, hidden], in place) += weight * y * rsqrt(mean(y^2) + eps), y [rows, hidden] float32
 // or `dtype`, or `slices` float32 partial sums [slices, rows, hidden].  Then mode 1: out = next_weight * x *
@@ -199,9 +204,50 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
                        int heads, int dim, int vdim, int chunked, int total_tokens, float* scratch, int64_t scratch_floats,
                        hipStream_t stream);
 
-// out[t, h, :] = retained[t, h, :] / rms(retained[t, h, :]) * silu(projected[t, gate_offset + h * vdim + :]).
+// out[t * out_row + h * vdim + :] = retained[t, h, :] / rms(retained[t, h, :]) * norm_weight * silu(projected[t,
+// gate_offset + h * vdim + :]) * out_scale; norm_weight [vdim] is shared by the heads (null: none).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
-                       int tokens, int heads, int vdim, float eps, hipStream_t stream);
+                       int tokens, int heads, int vdim, float eps, const void* norm_weight, int weight_is_f32,
+                       float out_scale, int64_t out_row, hipStream_t stream);
+
+// out[t] = (add_input ? h[t] : 0) + a causal convolution over the entry's inputs of `taps` taps per channel (weight
+// [width, taps], the last tap on the token itself); the taps - 1 inputs before a step are carried in `state`
+// [state_rows, taps - 1, width] float32 (row read_rows[entry], zeros where q_starts[entry] == 0) and the newest are
+// left in row write_rows[entry].
+int mlr_short_conv(const void* h, const void* weight, int weight_is_f32, float* state, int state_rows,
+                   const int* read_rows, const int* write_rows, const int* token_entry, const int* cu_q,
+                   const int* q_starts, void* out, int dtype, int tokens, int width, int taps, int add_input,
+                   hipStream_t stream);
+
+// projected [tokens, width] float32: q (heads * dim), k (kv_heads * dim), v (kv_heads * vdim), (gated) heads gate
+// logits.  q and k normed over their whole projection (weights q_norm, k_norm or null), rotated (two halves of the
+// first rotary_dim dims of a head), q times head_scale[head] into q_out [tokens, heads * head_dim], k and v into the
+// pages at slots[t] (heads padded with zeros to head_dim), gate = sigmoid(logits) float32 [tokens, heads].
+int mlr_qk_norm_rope_write(const float* projected, int width, const void* q_norm, const void* k_norm, int weight_is_f32,
+                           float eps, const float* head_scale, const float* cos_t, const float* sin_t, int rotary_dim,
+                           const int* slots, void* key_pages, void* value_pages, void* q_out, float* gate, int dtype,
+                           int tokens, int heads, int kv_heads, int dim, int vdim, int head_dim, int block_size,
+                           int num_pages, int gated, hipStream_t stream);
+
+// Tokens with pooled_slots[t] >= 0 complete a run of `pool` positions: the means of the run's keys and values, read
+// from the token pages through the block table, go to that slot of the pooled pages.
+int mlr_pool_kv_write(const void* key_pages, const void* value_pages, const int* block_table, int table_width,
+                      int num_pages, const int* token_entry, const int* positions, const int* pooled_slots,
+                      void* pooled_keys, void* pooled_values, int pooled_pages, int dtype, int tokens, int kv_heads,
+                      int head_dim, int block_size, int pool, hipStream_t stream);
+
+// out[t * out_row + head * out_dim + j] = attended[t, head * head_dim + j] * gate[t, head] * scale, j < out_dim.
+int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t out_row, int dtype, int tokens, int heads,
+                    int head_dim, int out_dim, float scale, hipStream_t stream);
+
+// Linear attention with a decay per key channel and token: decay = sigmoid(W2 low + bias)^(1 / tau) with `low` the
+// `rank` columns of `projected` from low_offset on (left in `decay` [tokens, heads * dim]); S = diag(decay) S + k v^T,
+// o = S^T (q * q_scale) per head; q, k, v are the leading columns of `projected` (float32).  State rows as for
+// mlr_retention_scan.
+int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, const void* decay_weight,
+                 const void* decay_bias, int weight_is_f32, int bias_is_f32, float tau, float* decay, float* state,
+                 int state_rows, const int* read_rows, const int* write_rows, const int* cu_q, const int* q_starts,
+                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, hipStream_t stream);
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds

@@ -22,7 +22,8 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const T* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ token_entry, const int* __restrict__ positions, T* __restrict__ out, int entries,
     int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, const T* __restrict__ pooled_keys, const T* __restrict__ pooled_values,
+    const int* __restrict__ pooled_table, int pooled_width, int pooled_pages, int pool) {
   __shared__ float qs[MAXD];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
@@ -44,7 +45,6 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   for (int i = lane; i < head_dim; i += kWave) qs[i] = to_f32(qrow[i]) * scale;
   __syncthreads();
 
-  const int* table = block_table + static_cast<int64_t>(entry) * table_width;
   const int first = first_visible_key(p, window, chunk);
   float m = -INFINITY;
   float l = 0.f;
@@ -53,50 +53,63 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   for (int j = 0; j < MAXD / kWave; ++j) acc[j] = 0.f;
   bool bad = false;
 
-  for (int k0 = first; k0 <= p; k0 += kWave) {
-    const int kpos = k0 + lane;
-    float s = -INFINITY;
-    int64_t off = -1;
-    int64_t voff = -1;
-    if (kpos <= p) {
-      const int logical = kpos / block_size;
-      const int page = logical < table_width ? table[logical] : -1;
-      if (page < 0 || page >= num_pages) {
-        bad = true;
-      } else {
-        const int in_page = kpos - logical * block_size;
-        const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + kvh) * block_size * head_dim;
-        off = head_base + static_cast<int64_t>(in_page) * head_dim;  // keys: [offset][dim]
-        voff = head_base + in_page;                                   // values: [dim][offset]
-        const T* kp = key_pages + off;
-        float dot = 0.f;
-        for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32(kp[i]), dot);
-        s = dot;
+  // Two sources share the one softmax: pooled entries (one key and value per run of `pool`
+  // positions that lies wholly before the window: entry b covers b * pool .. b * pool + pool - 1 and is
+  // seen when its last position is <= p - window), then the tokens first..p themselves.
+  const int pooled_seen = (pool > 0 && window > 0 && p - window >= 0) ? (p - window + 1) / pool : 0;
+  for (int source = 0; source < 2; ++source) {
+    const T* kpages = source == 0 ? pooled_keys : key_pages;
+    const T* vpages = source == 0 ? pooled_values : value_pages;
+    const int* table = (source == 0 ? pooled_table : block_table) + static_cast<int64_t>(entry) * (source == 0 ? pooled_width : table_width);
+    const int tw = source == 0 ? pooled_width : table_width;
+    const int np = source == 0 ? pooled_pages : num_pages;
+    const int begin = source == 0 ? 0 : first;
+    const int last = source == 0 ? pooled_seen - 1 : p;
+    for (int k0 = begin; k0 <= last; k0 += kWave) {
+      const int kpos = k0 + lane;
+      float s = -INFINITY;
+      int64_t off = -1;
+      int64_t voff = -1;
+      if (kpos <= last) {
+        const int logical = kpos / block_size;
+        const int page = logical < tw ? table[logical] : -1;
+        if (page < 0 || page >= np) {
+          bad = true;
+        } else {
+          const int in_page = kpos - logical * block_size;
+          const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + kvh) * block_size * head_dim;
+          off = head_base + static_cast<int64_t>(in_page) * head_dim;  // keys: [offset][dim]
+          voff = head_base + in_page;                                   // values: [dim][offset]
+          const T* kp = kpages + off;
+          float dot = 0.f;
+          for (int i = 0; i < head_dim; ++i) dot = fmaf(qs[i], to_f32(kp[i]), dot);
+          s = dot;
+        }
       }
-    }
-    const float m_new = fmaxf(m, wave_max(s));
-    const float pr = (off >= 0) ? expf(s - m_new) : 0.f;
-    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
-    l = l * alpha + wave_sum(pr);
-    m = m_new;
-    ps[lane] = pr;
-    offs[lane] = off;
-    voffs[lane] = voff;
-    __syncthreads();
-    const int count = min(kWave, p - k0 + 1);
+      const float m_new = fmaxf(m, wave_max(s));
+      const float pr = (off >= 0) ? expf(s - m_new) : 0.f;
+      const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+      l = l * alpha + wave_sum(pr);
+      m = m_new;
+      ps[lane] = pr;
+      offs[lane] = off;
+      voffs[lane] = voff;
+      __syncthreads();
+      const int count = min(kWave, last - k0 + 1);
 #pragma unroll
-    for (int j = 0; j < MAXD / kWave; ++j) acc[j] *= alpha;
-    for (int i = 0; i < count; ++i) {
-      if (offs[i] < 0) continue;
-      const float pi = ps[i];
-      const T* vp = value_pages + voffs[i];
+      for (int j = 0; j < MAXD / kWave; ++j) acc[j] *= alpha;
+      for (int i = 0; i < count; ++i) {
+        if (offs[i] < 0) continue;
+        const float pi = ps[i];
+        const T* vp = vpages + voffs[i];
 #pragma unroll
-      for (int j = 0; j < MAXD / kWave; ++j) {
-        const int dim = lane + j * kWave;
-        if (dim < head_dim) acc[j] = fmaf(pi, to_f32(vp[static_cast<int64_t>(dim) * block_size]), acc[j]);
+        for (int j = 0; j < MAXD / kWave; ++j) {
+          const int dim = lane + j * kWave;
+          if (dim < head_dim) acc[j] = fmaf(pi, to_f32(vp[static_cast<int64_t>(dim) * block_size]), acc[j]);
+        }
       }
+      __syncthreads();
     }
-    __syncthreads();
   }
 
   // a sink: one more term exp(sink) of the denominator, with no key and no value
@@ -126,7 +139,9 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
                                           const int* token_entry, const int* positions, void* out, int dtype,
                                           int tokens, int entries, int heads, int kv_heads, int head_dim,
                                           int block_size, int num_pages, float scale, int window, int chunk,
-                                          const float* sinks, hipStream_t stream) {
+                                          const float* sinks, const void* pooled_keys, const void* pooled_values,
+                                          const int* pooled_table, int pooled_width, int pooled_pages, int pool,
+                                          hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && token_entry && positions && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && kv_heads > 0, "sizes must be > 0");
   MLR_REQUIRE(heads % kv_heads == 0, "query heads must be a multiple of KV heads");
@@ -136,13 +151,17 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
   MLR_REQUIRE(scale > 0.f && scale < INFINITY, "scale must be positive and finite");
   MLR_REQUIRE(window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0), "a window or a chunked mask, each >= 0");
   MLR_REQUIRE(heads < 65536, "too many heads for one launch");
+  MLR_REQUIRE(pool >= 0 && (pool == 0 || (window > 0 && pooled_keys && pooled_values && pooled_table && pooled_width > 0 &&
+                                          pooled_pages > 0)),
+              "pooled entries need a window, their pages and their table");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   dim3 grid(tokens, heads);
 #define MLR_SIMPLE(T, MAXD)                                                                                      \
   paged_attention_simple_kernel<T, MAXD><<<grid, kWave, 0, stream>>>(                                            \
       static_cast<const T*>(q), q_stride, static_cast<const T*>(key_pages), static_cast<const T*>(value_pages),   \
       block_table, table_width, token_entry, positions, static_cast<T*>(out), entries, heads, kv_heads, head_dim, \
-      block_size, num_pages, scale, window, chunk, sinks)
+      block_size, num_pages, scale, window, chunk, sinks, static_cast<const T*>(pooled_keys),                    \
+      static_cast<const T*>(pooled_values), pooled_table, pooled_width, pooled_pages, pool)
   if (head_dim > 256) {
     if (dtype == kF32)
       MLR_SIMPLE(float, kMaxHeadDim);
@@ -156,13 +175,15 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
         static_cast<const float*>(q), q_stride, static_cast<const float*>(key_pages),
         static_cast<const float*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
-        sinks);
+        sinks, static_cast<const float*>(pooled_keys), static_cast<const float*>(pooled_values), pooled_table,
+        pooled_width, pooled_pages, pool);
   else
     paged_attention_simple_kernel<bf16, 256><<<grid, kWave, 0, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
         static_cast<const bf16*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
-        sinks);
+        sinks, static_cast<const bf16*>(pooled_keys), static_cast<const bf16*>(pooled_values), pooled_table,
+        pooled_width, pooled_pages, pool);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -754,12 +754,16 @@ __global__ __launch_bounds__(256) void retention_apply_kernel(const float* __res
   }
 }
 
-// out[t, h, :] = o / sqrt(mean(o^2) + eps) * silu(z), o = retained[t, h, :] (float32), z = the gate sums at
-// column gate_offset + h * vdim of p [tokens, width] (float32).  One wavefront per (token, head).
+// out[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(z) * out_scale, o = retained[t, h, :] (float32), z = the gate
+// sums at column gate_offset + h * vdim of p [tokens, width] (float32), w [vdim] a weight that all heads share
+// (null: none).  A row of `out` is out_row elements long and the heads start at its column 0.  One wavefront
+// per (token, head).
 template <typename T>
 __global__ __launch_bounds__(64) void retention_gate_kernel(const float* __restrict__ retained,
                                                             const float* __restrict__ p, int width, int gate_offset,
-                                                            T* __restrict__ out, int heads, int vdim, float eps) {
+                                                            T* __restrict__ out, int64_t out_row, int heads, int vdim,
+                                                            float eps, const void* __restrict__ norm_weight,
+                                                            int weight_is_f32, float out_scale) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   const float* o = retained + (t * heads + h) * vdim;
@@ -767,10 +771,12 @@ __global__ __launch_bounds__(64) void retention_gate_kernel(const float* __restr
   for (int i = threadIdx.x; i < vdim; i += 64) ss += o[i] * o[i];
   const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
   const float* z = p + t * width + gate_offset + static_cast<int64_t>(h) * vdim;
-  T* dst = out + (t * heads + h) * vdim;
+  T* dst = out + t * out_row + static_cast<int64_t>(h) * vdim;
   for (int i = threadIdx.x; i < vdim; i += 64) {
     const float zv = z[i];
-    dst[i] = from_f32<T>((o[i] * inv) * (zv / (1.0f + expf(-zv))));
+    float normed = o[i] * inv;
+    if (norm_weight != nullptr) normed *= load_as_f32(norm_weight, i, weight_is_f32);
+    dst[i] = from_f32<T>(normed * (zv / (1.0f + expf(-zv))) * out_scale);
   }
 }
 
@@ -968,18 +974,22 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
 }
 
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
-                       int tokens, int heads, int vdim, float eps, hipStream_t stream) {
+                       int tokens, int heads, int vdim, float eps, const void* norm_weight, int weight_is_f32,
+                       float out_scale, int64_t out_row, hipStream_t stream) {
   MLR_REQUIRE(retained && projected && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && heads > 0 && heads < 65536 && vdim > 0, "sizes must be > 0");
   MLR_REQUIRE(gate_offset >= 0 && width >= gate_offset + heads * vdim, "the projected rows do not hold the gate");
+  MLR_REQUIRE(out_row >= static_cast<int64_t>(heads) * vdim, "a row of the output is shorter than the heads");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   dim3 grid(tokens, heads);
   if (dtype == kF32)
     retention_gate_kernel<float><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
-                                                          static_cast<float*>(out), heads, vdim, eps);
+                                                          static_cast<float*>(out), out_row, heads, vdim, eps,
+                                                          norm_weight, weight_is_f32, out_scale);
   else
     retention_gate_kernel<bf16><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
-                                                         static_cast<bf16*>(out), heads, vdim, eps);
+                                                         static_cast<bf16*>(out), out_row, heads, vdim, eps,
+                                                         norm_weight, weight_is_f32, out_scale);
   MLR_LAUNCH_CHECK();
   return 0;
 }

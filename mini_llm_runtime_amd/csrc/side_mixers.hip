@@ -1,0 +1,417 @@
+// Kernels of mixers that run side by side on one input: a short causal convolution with carried
+// inputs, queries and keys normed over their whole projection, rotated and stored, pooled entries of
+// the key/value cache, a gate per head, and linear attention with a decay per key channel and token.
+#include "api.h"
+#include "common.h"
+
+namespace mlr {
+namespace {
+
+// out[t, c] = h[t, c] + sum_j w[c, j] * in(t - (taps - 1) + j), in() = the entry's inputs in order: those
+// of this step, before them the `taps - 1` inputs that the state row read_rows[entry] carries
+// ([rows, taps - 1, width] float32, the oldest first; zeros where the entry starts its request or the
+// request is shorter).  The entry's last token leaves the newest taps - 1 inputs in row write_rows[entry].
+// Sums in float32, one rounding.  A workgroup per token, threads over the channels.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_kernel(const T* __restrict__ h, const void* __restrict__ weight,
+                                                         int weight_is_f32, float* __restrict__ state,
+                                                         const int* __restrict__ read_rows,
+                                                         const int* __restrict__ write_rows,
+                                                         const int* __restrict__ token_entry,
+                                                         const int* __restrict__ cu_q, const int* __restrict__ q_starts,
+                                                         T* __restrict__ out, int width, int taps, int add_input) {
+  const int64_t t = blockIdx.x;
+  const int entry = token_entry[t];
+  const int first = cu_q[entry];
+  const int end = cu_q[entry + 1];
+  const int i = static_cast<int>(t) - first;  // place among the step's tokens of the entry
+  const int carried = taps - 1;
+  const bool fresh = q_starts[entry] == 0;
+  const float* old = state + static_cast<int64_t>(read_rows[entry]) * carried * width;
+  auto input = [&](int idx, int c) -> float {  // idx counts from the step's first token of the entry
+    if (idx >= 0) return to_f32(h[(static_cast<int64_t>(first) + idx) * width + c]);
+    if (fresh) return 0.f;
+    return old[static_cast<int64_t>(carried + idx) * width + c];
+  };
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = add_input ? to_f32(h[t * width + c]) : 0.f;
+    for (int j = 0; j < taps; ++j)
+      acc = fmaf(load_as_f32(weight, static_cast<int64_t>(c) * taps + j, weight_is_f32), input(i - carried + j, c), acc);
+    out[t * width + c] = from_f32<T>(acc);
+  }
+  if (static_cast<int>(t) == end - 1 && carried > 0) {
+    const int n = end - first;
+    float* dst = state + static_cast<int64_t>(write_rows[entry]) * carried * width;
+    for (int c = threadIdx.x; c < width; c += 256)
+      for (int s = 0; s < carried; ++s) dst[static_cast<int64_t>(s) * width + c] = input(n - carried + s, c);
+  }
+}
+
+// One token's projected row p[t] (float32): q (heads * dim), k (kv_heads * dim), v (kv_heads * vdim),
+// then (gated) one gate logit per head.
+//  * q and k are each divided by the root mean square over their WHOLE projection and multiplied by a
+//    weight of that size (q_norm, k_norm; null: no norm),
+//  * the first `rdims` dims of every head turn in two halves (pair j, j + rdims / 2) by cos/sin[t],
+//  * q times head_scale[head] (null: 1) goes to q_out [tokens, heads * D], k and v to slot[t] of the key pages
+//    [page, kv_head, offset, D] and the value pages [page, kv_head, D, offset]; dims beyond dim / vdim are
+//    zeros; a negative slot stores nothing,
+//  * gate[t, head] = sigmoid(logit), float32.
+// Everything in float32, one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
+    const float* __restrict__ p, int width, const void* __restrict__ q_norm, const void* __restrict__ k_norm,
+    int weight_is_f32, float eps, const float* __restrict__ head_scale, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int rdims, const int* __restrict__ slots, T* __restrict__ key_pages,
+    T* __restrict__ value_pages, T* __restrict__ q_out, float* __restrict__ gate, int heads, int kv_heads, int dim,
+    int vdim, int D, int block_size, int num_pages, int gated) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const float* q = p + t * width;
+  const float* k = q + heads * dim;
+  const float* v = k + kv_heads * dim;
+  const int half = rdims / 2;
+  const float* cs = cos_t ? cos_t + t * half : nullptr;
+  const float* sn = sin_t ? sin_t + t * half : nullptr;
+  float q_inv = 1.f, k_inv = 1.f;
+  if (q_norm != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < heads * dim; i += 256) ss += q[i] * q[i];
+    q_inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(heads * dim) + eps);
+  }
+  if (k_norm != nullptr) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < kv_heads * dim; i += 256) ss += k[i] * k[i];
+    k_inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(kv_heads * dim) + eps);
+  }
+  // dim j of head `head` of a normed, rotated projection
+  auto turned = [&](const float* part, const void* w, float inv, int head, int j) -> float {
+    const int at = head * dim + j;
+    auto normed = [&](int idx) { return w ? (part[idx] * inv) * load_as_f32(w, idx, weight_is_f32) : part[idx]; };
+    if (j >= rdims || cs == nullptr) return normed(at);
+    return j < half ? normed(at) * cs[j] - normed(at + half) * sn[j]
+                    : normed(at) * cs[j - half] + normed(at - half) * sn[j - half];
+  };
+  for (int i = threadIdx.x; i < heads * D; i += 256) {
+    const int hd = i / D;
+    const int j = i - hd * D;
+    float val = 0.f;
+    if (j < dim) {
+      val = turned(q, q_norm, q_inv, hd, j);
+      if (head_scale != nullptr) val *= head_scale[hd];
+    }
+    q_out[t * heads * D + i] = from_f32<T>(val);
+  }
+  const int slot = slots[t];
+  if (slot >= 0) {
+    const int page = slot / block_size;
+    const int off = slot - page * block_size;
+    if (page < num_pages) {
+      for (int i = threadIdx.x; i < kv_heads * D; i += 256) {
+        const int g = i / D;
+        const int j = i - g * D;
+        const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + g) * block_size * D;
+        key_pages[head_base + static_cast<int64_t>(off) * D + j] = from_f32<T>(j < dim ? turned(k, k_norm, k_inv, g, j) : 0.f);
+        value_pages[head_base + static_cast<int64_t>(j) * block_size + off] = from_f32<T>(j < vdim ? v[g * vdim + j] : 0.f);
+      }
+    }
+  }
+  if (gated) {
+    const float* logits = v + kv_heads * vdim;
+    for (int hd = threadIdx.x; hd < heads; hd += 256) gate[t * heads + hd] = 1.0f / (1.0f + expf(-logits[hd]));
+  }
+}
+
+// A token that completes a run of `pool` positions (pooled_slots[t] >= 0; its position p is the run's
+// last) stores the means of the run's keys and of its values, as the token pages hold them, at that
+// slot of the pooled pages (same layouts).  Sums in float32 in the order of the positions.
+// Grid (tokens, kv_heads).
+template <typename T>
+__global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__ key_pages,
+                                                           const T* __restrict__ value_pages,
+                                                           const int* __restrict__ block_table, int table_width,
+                                                           int num_pages, const int* __restrict__ token_entry,
+                                                           const int* __restrict__ positions,
+                                                           const int* __restrict__ pooled_slots,
+                                                           T* __restrict__ pooled_keys, T* __restrict__ pooled_values,
+                                                           int pooled_pages, int kv_heads, int D, int block_size,
+                                                           int pool) {
+  const int t = blockIdx.x;
+  const int slot = pooled_slots[t];
+  if (slot < 0) return;
+  const int g = blockIdx.y;
+  const int p = positions[t];
+  const int* table = block_table + static_cast<int64_t>(token_entry[t]) * table_width;
+  const int dst_page = slot / block_size;
+  const int dst_off = slot - dst_page * block_size;
+  if (dst_page >= pooled_pages || p - pool + 1 < 0) return;
+  const float inv = 1.0f / static_cast<float>(pool);
+  const int64_t dst_base = (static_cast<int64_t>(dst_page) * kv_heads + g) * block_size * D;
+  for (int i = threadIdx.x; i < D; i += 64) {
+    float ks = 0.f, vs = 0.f;
+    for (int j = p - pool + 1; j <= p; ++j) {
+      const int logical = j / block_size;
+      const int page = logical < table_width ? table[logical] : -1;
+      if (page < 0 || page >= num_pages) {
+        ks = vs = NAN;  // a run whose tokens are gone cannot be pooled: show it
+        break;
+      }
+      const int off = j - logical * block_size;
+      const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + g) * block_size * D;
+      ks += to_f32(key_pages[head_base + static_cast<int64_t>(off) * D + i]);
+      vs += to_f32(value_pages[head_base + static_cast<int64_t>(i) * block_size + off]);
+    }
+    pooled_keys[dst_base + static_cast<int64_t>(dst_off) * D + i] = from_f32<T>(ks * inv);
+    pooled_values[dst_base + static_cast<int64_t>(i) * block_size + dst_off] = from_f32<T>(vs * inv);
+  }
+}
+
+// out[t, column + head * out_dim + j] = attended[t, head * D + j] * gate[t, head] * scale for j < out_dim; gate
+// float32 [tokens, heads] (null: 1); a row of `out` is out_row elements long.
+template <typename T>
+__global__ __launch_bounds__(256) void scale_heads_kernel(const T* __restrict__ attended, const float* __restrict__ gate,
+                                                          T* __restrict__ out, int64_t out_row, int heads, int D,
+                                                          int out_dim, float scale) {
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < heads * out_dim; i += 256) {
+    const int hd = i / out_dim;
+    const int j = i - hd * out_dim;
+    float val = to_f32(attended[(t * heads + hd) * D + j]) * scale;
+    if (gate != nullptr) val *= gate[t * heads + hd];
+    out[t * out_row + i] = from_f32<T>(val);
+  }
+}
+
+// decay[t, c] = sigmoid(z)^(1 / tau), z = sum_r w2[c, r] * low[t, r] + bias[c]: `low` are `rank` columns of
+// the projected rows p (float32) from column low_offset on, w2 [channels, rank], all sums in float32.
+// log sigmoid(z) = -softplus(-z), taken on the side where the exponential is small.
+__global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict__ p, int width, int low_offset, int rank,
+                                                        const void* __restrict__ w2, const void* __restrict__ bias,
+                                                        int weight_is_f32, int bias_is_f32, float inv_tau,
+                                                        float* __restrict__ decay, int channels) {
+  extern __shared__ float low[];
+  const int64_t t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += 256) low[r] = p[t * width + low_offset + r];
+  __syncthreads();
+  for (int c = threadIdx.x; c < channels; c += 256) {
+    float z = bias ? load_as_f32(bias, c, bias_is_f32) : 0.f;
+    for (int r = 0; r < rank; ++r) z = fmaf(load_as_f32(w2, static_cast<int64_t>(c) * rank + r, weight_is_f32), low[r], z);
+    const float log_sigmoid = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+    decay[t * channels + c] = expf(log_sigmoid * inv_tau);
+  }
+}
+
+// S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t * q_scale) per (entry, head), the entry's tokens in
+// order; a_t [dim] from `decay` [tokens, heads * dim].  `p` [tokens, width] float32 holds q (heads * dim), k
+// (heads * dim), v (heads * vdim).  A wavefront owns 16 columns of one head's state: lane = (group of dims g =
+// lane / 16, column c = lane % 16) keeps S[d][c] for d = 4 i + g in registers; tokens go through LDS kBatch at
+// a time.  State rows as for the other recurrent kernels: read_rows[entry] (zeros when the entry starts its
+// request) to write_rows[entry]; out [tokens, heads * vdim] float32.
+constexpr int kGlaBatch = 8;
+
+template <int DPL>
+__global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ p, int width,
+                                                      const float* __restrict__ decay, float* __restrict__ state,
+                                                      const int* __restrict__ read_rows,
+                                                      const int* __restrict__ write_rows, const int* __restrict__ cu_q,
+                                                      const int* __restrict__ q_starts, float q_scale,
+                                                      float* __restrict__ out, int heads, int dim, int vdim) {
+  __shared__ float qs[kGlaBatch][4 * DPL];
+  __shared__ float ks[kGlaBatch][4 * DPL];
+  __shared__ float as[kGlaBatch][4 * DPL];
+  __shared__ float vs[kGlaBatch][16];
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int v0 = blockIdx.z * 16;
+  const int lane = threadIdx.x;
+  const int g = lane / 16;
+  const int c = lane % 16;
+  const bool column = v0 + c < vdim;
+  const int t_first = cu_q[entry];
+  const int t_end = cu_q[entry + 1];
+  const int64_t head_state = static_cast<int64_t>(dim) * vdim;
+
+  float S[DPL];
+  const bool carried = q_starts[entry] > 0;
+  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = 4 * i + g;
+    S[i] = (carried && column && d < dim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+  }
+  for (int tb = t_first; tb < t_end; tb += kGlaBatch) {
+    const int count = min(kGlaBatch, t_end - tb);
+    __syncthreads();  // the batch before is done with
+    for (int idx = lane; idx < count * dim; idx += 64) {
+      const int u = idx / dim;
+      const int d = idx - u * dim;
+      const int64_t t = tb + u;
+      const float* q = p + t * width + static_cast<int64_t>(h) * dim;
+      qs[u][d] = q[d] * q_scale;
+      ks[u][d] = q[static_cast<int64_t>(heads) * dim + d];
+      as[u][d] = decay[(t * heads + h) * dim + d];
+    }
+    for (int idx = lane; idx < count * 16; idx += 64) {
+      const int u = idx / 16;
+      const int cc = idx - u * 16;
+      vs[u][cc] = v0 + cc < vdim
+                      ? p[static_cast<int64_t>(tb + u) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v0 + cc]
+                      : 0.f;
+    }
+    __syncthreads();
+    for (int u = 0; u < count; ++u) {
+      const float vv = vs[u][c];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = 4 * i + g;
+        if (d < dim) {
+          S[i] = fmaf(as[u][d], S[i], ks[u][d] * vv);
+          o = fmaf(S[i], qs[u][d], o);
+        }
+      }
+      o += __shfl_xor(o, 16, kWave);
+      o += __shfl_xor(o, 32, kWave);
+      if (g == 0 && column) out[static_cast<int64_t>(tb + u) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + c] = o;
+    }
+  }
+  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = 4 * i + g;
+    if (column && d < dim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = S[i];
+  }
+}
+
+}  // namespace
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+int mlr_short_conv(const void* h, const void* weight, int weight_is_f32, float* state, int state_rows,
+                   const int* read_rows, const int* write_rows, const int* token_entry, const int* cu_q,
+                   const int* q_starts, void* out, int dtype, int tokens, int width, int taps, int add_input,
+                   hipStream_t stream) {
+  MLR_REQUIRE(h && weight && read_rows && write_rows && token_entry && cu_q && q_starts && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && width > 0 && taps > 0, "sizes must be > 0");
+  MLR_REQUIRE(taps == 1 || (state != nullptr && state_rows > 0), "carried inputs need a state");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    short_conv_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(h), weight, weight_is_f32, state,
+                                                         read_rows, write_rows, token_entry, cu_q, q_starts,
+                                                         static_cast<float*>(out), width, taps, add_input);
+  else
+    short_conv_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(h), weight, weight_is_f32, state,
+                                                        read_rows, write_rows, token_entry, cu_q, q_starts,
+                                                        static_cast<bf16*>(out), width, taps, add_input);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_qk_norm_rope_write(const float* projected, int width, const void* q_norm, const void* k_norm, int weight_is_f32,
+                           float eps, const float* head_scale, const float* cos_t, const float* sin_t, int rotary_dim,
+                           const int* slots, void* key_pages, void* value_pages, void* q_out, float* gate, int dtype,
+                           int tokens, int heads, int kv_heads, int dim, int vdim, int head_dim, int block_size,
+                           int num_pages, int gated, hipStream_t stream) {
+  MLR_REQUIRE(projected && slots && key_pages && value_pages && q_out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "sizes must be > 0");
+  MLR_REQUIRE(head_dim >= dim && head_dim >= vdim, "the pages' head size must hold keys and values");
+  MLR_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= dim, "rotary_dim must be even and within dim");
+  MLR_REQUIRE(rotary_dim == 0 || (cos_t && sin_t), "a rotation needs its tables");
+  MLR_REQUIRE(!gated || gate, "gates need their output");
+  MLR_REQUIRE(width >= heads * dim + kv_heads * (dim + vdim) + (gated ? heads : 0), "the projected rows are too narrow");
+  MLR_REQUIRE(block_size > 0 && num_pages > 0, "pages must exist");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    qk_norm_rope_write_kernel<float><<<tokens, 256, 0, stream>>>(
+        projected, width, q_norm, k_norm, weight_is_f32, eps, head_scale, rotary_dim ? cos_t : nullptr,
+        rotary_dim ? sin_t : nullptr, rotary_dim, slots, static_cast<float*>(key_pages), static_cast<float*>(value_pages),
+        static_cast<float*>(q_out), gate, heads, kv_heads, dim, vdim, head_dim, block_size, num_pages, gated);
+  else
+    qk_norm_rope_write_kernel<bf16><<<tokens, 256, 0, stream>>>(
+        projected, width, q_norm, k_norm, weight_is_f32, eps, head_scale, rotary_dim ? cos_t : nullptr,
+        rotary_dim ? sin_t : nullptr, rotary_dim, slots, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages),
+        static_cast<bf16*>(q_out), gate, heads, kv_heads, dim, vdim, head_dim, block_size, num_pages, gated);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_pool_kv_write(const void* key_pages, const void* value_pages, const int* block_table, int table_width,
+                      int num_pages, const int* token_entry, const int* positions, const int* pooled_slots,
+                      void* pooled_keys, void* pooled_values, int pooled_pages, int dtype, int tokens, int kv_heads,
+                      int head_dim, int block_size, int pool, hipStream_t stream) {
+  MLR_REQUIRE(key_pages && value_pages && block_table && token_entry && positions && pooled_slots && pooled_keys &&
+                  pooled_values,
+              "null pointer");
+  MLR_REQUIRE(tokens > 0 && kv_heads > 0 && kv_heads < 65536 && head_dim > 0 && block_size > 0 && pool > 0,
+              "sizes must be > 0");
+  MLR_REQUIRE(table_width > 0 && num_pages > 0 && pooled_pages > 0, "pages must exist");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  dim3 grid(tokens, kv_heads);
+  if (dtype == kF32)
+    pool_kv_write_kernel<float><<<grid, 64, 0, stream>>>(
+        static_cast<const float*>(key_pages), static_cast<const float*>(value_pages), block_table, table_width, num_pages,
+        token_entry, positions, pooled_slots, static_cast<float*>(pooled_keys), static_cast<float*>(pooled_values),
+        pooled_pages, kv_heads, head_dim, block_size, pool);
+  else
+    pool_kv_write_kernel<bf16><<<grid, 64, 0, stream>>>(
+        static_cast<const bf16*>(key_pages), static_cast<const bf16*>(value_pages), block_table, table_width, num_pages,
+        token_entry, positions, pooled_slots, static_cast<bf16*>(pooled_keys), static_cast<bf16*>(pooled_values),
+        pooled_pages, kv_heads, head_dim, block_size, pool);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t out_row, int dtype, int tokens, int heads,
+                    int head_dim, int out_dim, float scale, hipStream_t stream) {
+  MLR_REQUIRE(attended && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && head_dim > 0 && out_dim > 0 && out_dim <= head_dim, "sizes must be > 0");
+  MLR_REQUIRE(out_row >= static_cast<int64_t>(heads) * out_dim, "a row of the output is shorter than the heads");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    scale_heads_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(attended), gate,
+                                                          static_cast<float*>(out), out_row, heads, head_dim, out_dim,
+                                                          scale);
+  else
+    scale_heads_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(attended), gate,
+                                                         static_cast<bf16*>(out), out_row, heads, head_dim, out_dim,
+                                                         scale);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, const void* decay_weight,
+                 const void* decay_bias, int weight_is_f32, int bias_is_f32, float tau, float* decay, float* state,
+                 int state_rows, const int* read_rows, const int* write_rows, const int* cu_q, const int* q_starts,
+                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, hipStream_t stream) {
+  MLR_REQUIRE(projected && decay_weight && decay && state && read_rows && write_rows && cu_q && q_starts && out,
+              "null pointer");
+  MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0,
+              "sizes must be > 0");
+  MLR_REQUIRE(rank > 0 && rank <= 4096 && low_offset >= 0 && width >= low_offset + rank, "the projected rows do not hold the decay's inputs");
+  MLR_REQUIRE(width >= 2 * heads * dim + heads * vdim, "the projected rows do not hold q, k and v");
+  MLR_REQUIRE(tau > 0.f, "tau must be > 0");
+  MLR_REQUIRE(dim <= 256, "heads of up to 256 dims");
+  gla_decay_kernel<<<tokens, 256, rank * sizeof(float), stream>>>(projected, width, low_offset, rank, decay_weight,
+                                                                  decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau, decay,
+                                                                  heads * dim);
+  MLR_LAUNCH_CHECK();
+  dim3 grid(entries, heads, (vdim + 15) / 16);
+#define MLR_GLA(DPL)                                                                                              \
+  gla_scan_kernel<DPL><<<grid, 64, 0, stream>>>(projected, width, decay, state, read_rows, write_rows, cu_q,      \
+                                                q_starts, q_scale, out, heads, dim, vdim)
+  if (dim <= 32)
+    MLR_GLA(8);
+  else if (dim <= 64)
+    MLR_GLA(16);
+  else if (dim <= 128)
+    MLR_GLA(32);
+  else
+    MLR_GLA(64);
+#undef MLR_GLA
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -66,6 +66,7 @@ CORE = Module(
         "attention_simple.hip",
         "moe.hip",
         "mixers.hip",
+        "side_mixers.hip",
         "sampling.hip",
     ),
 )

@@ -40,7 +40,17 @@ _SIGNATURES = {
         [_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _I, _VP, _I64, _VP], _I,
     ),
     "mlr_retention_scratch": ([_I, _I, _I, _I, _I], _I64),
-    "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP], _I),
+    "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP, _I, _F, _I64, _VP], _I),
+    "mlr_short_conv": ([_VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_qk_norm_rope_write": (
+        [_VP, _I, _VP, _VP, _I, _F, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        _I,
+    ),
+    "mlr_pool_kv_write": ([_VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_scale_heads": ([_VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _F, _VP], _I),
+    "mlr_gla_scan": (
+        [_VP, _I, _I, _I, _VP, _VP, _I, _I, _F, _VP, _VP, _I, _VP, _VP, _VP, _VP, _F, _VP, _I, _I, _I, _I, _I, _VP], _I,
+    ),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
     "mlr_scale_softcap": ([_VP, _F, _F, _I64, _VP], _I),
@@ -74,7 +84,8 @@ _SIGNATURES = {
     ),
     "mlr_gemm_merge_fused_bf16": ([_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP, _VP, _VP, _VP,
+         _I, _I, _I, _VP],
         _I,
     ),
     "mlr_sample": ([_VP, _VP, _VP, _VP, _VP, _I, _I, _VP], _I),
@@ -312,9 +323,14 @@ class HipOps:
         return out
 
     def add_(self, x: torch.Tensor, delta: torch.Tensor) -> None:
-        """x (float32) += delta (the engine's dtype, or float32), in place."""
+        """x (float32) += delta (the engine's dtype, or float32; or a float32 stack [S, ...] of partial sums, or a
+        product that has not run), in place."""
         self._check(x, "residual stream", torch.float32)
         delta = self.settle(delta)
+        if delta.dim() == x.dim() + 1:  # partial sums: one after the other, in order
+            for part in delta:
+                self.add_(x, part)
+            return
         self._check(delta, "residual delta", (self.dtype, torch.float32), tuple(x.shape))
         self._call("mlr_add", self._ptr(x), self._ptr(delta), _dtype_code(delta.dtype), x.numel(), self._stream())
 
@@ -877,8 +893,13 @@ class HipOps:
         plan: Any = None,
         chunk: Optional[int] = None,
         sinks: Optional[torch.Tensor] = None,
+        pooled: Optional[tuple] = None,
     ):
         """Causal attention of the step's tokens over their requests' pages.
+
+        pooled: (key pages, value pages, block table, pool) of a second set of pages that holds ONE key and
+        value for every run of `pool` positions (see `pool_kv_write`); with a window, a query at position p
+        then also sees the entries of the runs that end at or before p - window, in the same softmax.
 
         sinks: float32 [num_heads]; the softmax's denominator of head h then also holds exp(sinks[h]), a
         term with no key and no value (not scaled).
@@ -923,8 +944,21 @@ class HipOps:
             self._check(sinks, "sinks", torch.float32, (num_heads,))
         out = self._empty((tokens, num_heads * head_dim), self.dtype)
         width = block_table.shape[1]
+        pooled_keys = pooled_values = pooled_table = None
+        pooled_width = pooled_pages = pool = 0
+        if pooled is not None:
+            pooled_keys, pooled_values, pooled_table, pool = pooled
+            pool = int(pool)
+            if pool <= 0 or not window:
+                raise KernelError("pooled entries have a run length > 0 and come with a window")
+            pooled_pages = self._check_pages(pooled_keys, pooled_values, num_kv_heads, head_dim, block_size)
+            self._check(pooled_table, "pooled block table", torch.int32, (entries, None))
+            pooled_width = pooled_table.shape[1]
+            if pooled_width * block_size * pool < ctx.max_context_len - int(window) - pool + 1:
+                raise KernelError("the pooled block table is narrower than the runs before the longest context's window")
         use_mfma = (
             kernel == "auto"
+            and pooled is None
             and self.dtype == torch.bfloat16
             and head_dim % 16 == 0
             and 16 <= head_dim <= 256
@@ -945,7 +979,8 @@ class HipOps:
                 "mlr_paged_attention_simple", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
                 self._ptr(out), self.code, tokens, entries, num_heads, num_kv_heads, head_dim, block_size,
-                num_pages, float(scale), int(window or 0), chunk, self._ptr(sinks), self._stream(),
+                num_pages, float(scale), int(window or 0), chunk, self._ptr(sinks), self._ptr(pooled_keys),
+                self._ptr(pooled_values), self._ptr(pooled_table), pooled_width, pooled_pages, pool, self._stream(),
             )
             return out
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
@@ -1175,19 +1210,255 @@ class HipOps:
         return out
 
     def retention_gate(
-        self, retained: torch.Tensor, projected: torch.Tensor, *, heads: int, value_dim: int, gate_offset: int, eps: float
+        self,
+        retained: torch.Tensor,
+        projected: torch.Tensor,
+        *,
+        heads: int,
+        value_dim: int,
+        gate_offset: int,
+        eps: float,
+        norm_weight: Optional[torch.Tensor] = None,
+        scale: float = 1.0,
+        out: Optional[torch.Tensor] = None,
+        column: int = 0,
     ) -> torch.Tensor:
-        """Every head's retained[t, h, :] divided by its root mean square (eps inside the root), times silu of
-        the gate sums in columns gate_offset .. of `projected`; [T, heads * value_dim] in the engine's dtype."""
+        """Every head's retained[t, h, :] divided by its root mean square (eps inside the root), times
+        `norm_weight` [value_dim] (one weight for all heads; None: none), times silu of the gate sums in columns
+        gate_offset .. of `projected`, times `scale`; [T, heads * value_dim] in the engine's dtype, or written
+        into columns column .. of the wider `out` [T, K]."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
         self._check(retained, "retained", torch.float32, (tokens, heads * value_dim))
         if gate_offset < 0 or gate_offset + heads * value_dim > width:
             raise KernelError("the projected rows do not hold the gate")
-        out = self._empty((tokens, heads * value_dim), self.dtype)
+        if norm_weight is not None:
+            self._check(norm_weight, "head norm weight", (torch.float32, self.dtype), (value_dim,))
+        out, view, row = self._columns(out, column, tokens, heads * value_dim)
         self._call(
-            "mlr_retention_gate", self._ptr(retained), self._ptr(projected), width, int(gate_offset), self._ptr(out),
-            self.code, tokens, heads, value_dim, float(eps), self._stream(),
+            "mlr_retention_gate", self._ptr(retained), self._ptr(projected), width, int(gate_offset), view,
+            self.code, tokens, heads, value_dim, float(eps), self._ptr(norm_weight),
+            int(norm_weight is not None and norm_weight.dtype == torch.float32), float(scale), row, self._stream(),
+        )
+        return out
+
+    def _columns(self, out: Optional[torch.Tensor], column: int, tokens: int, width: int):
+        """Where a kernel writes [tokens, width] activations: a tensor of its own, or columns column ..
+        column + width of a wider `out`; returns (tensor, pointer to the first element, row length)."""
+        if out is None:
+            out = self._empty((tokens, width), self.dtype)
+            return out, self._ptr(out), width
+        self._check(out, "activations of several parts", self.dtype, (tokens, None))
+        row = out.shape[1]
+        if column < 0 or column + width > row:
+            raise KernelError("the columns lie outside the rows they are written into")
+        return out, _VP(out.data_ptr() + column * out.element_size()), row
+
+    # ---- parts that run side by side ---------------------------------------------------------------------
+    def short_conv(
+        self,
+        h: torch.Tensor,
+        weight: torch.Tensor,
+        state: Optional[torch.Tensor],
+        read_rows: Optional[torch.Tensor],
+        write_rows: Optional[torch.Tensor],
+        ctx: Any,
+        *,
+        add_input: bool = True,
+    ) -> torch.Tensor:
+        """h [T, W] (+ when `add_input`) its causal convolution over time, per channel and entry: out_t = sum_j
+        weight[:, j] * h_(t - taps + 1 + j), weight [W, taps].  The taps - 1 inputs before a step's first token
+        come from row read_rows[entry] of `state` [rows, taps - 1, W] float32 (zeros where the entry starts its
+        request); the newest taps - 1 inputs are left in row write_rows[entry]."""
+        self._check(h, "convolution input", self.dtype, (None, None))
+        tokens, width = h.shape
+        self._check(weight, "convolution taps", (torch.float32, self.dtype), (width, None))
+        taps = weight.shape[1]
+        entries = ctx.num_entries
+        rows = 0
+        if taps > 1:
+            self._check(state, "carried inputs", torch.float32, (None, taps - 1, width))
+            rows = state.shape[0]
+        else:
+            state = None
+            read_rows, write_rows = ctx.q_starts, ctx.q_starts  # never read
+        self._check(read_rows, "state rows to read", torch.int32, (entries,))
+        self._check(write_rows, "state rows to write", torch.int32, (entries,))
+        self._check(ctx.token_entry, "token entries", torch.int32, (tokens,))
+        self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
+        self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
+        out = self._empty((tokens, width), self.dtype)
+        self._call(
+            "mlr_short_conv", self._ptr(h), self._ptr(weight), int(weight.dtype == torch.float32), self._ptr(state), rows,
+            self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.token_entry), self._ptr(ctx.cu_q),
+            self._ptr(ctx.q_starts), self._ptr(out), self.code, tokens, width, taps, int(bool(add_input)), self._stream(),
+        )
+        return out
+
+    def qk_norm_rope_write(
+        self,
+        projected: torch.Tensor,
+        q_norm: Optional[torch.Tensor],
+        k_norm: Optional[torch.Tensor],
+        eps: float,
+        head_scale: Optional[torch.Tensor],
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        slot_mapping: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        *,
+        num_heads: int,
+        num_kv_heads: int,
+        dim: int,
+        value_dim: int,
+        head_dim: int,
+        block_size: int,
+        gated: bool = False,
+    ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """From the float32 sums `projected` [T, q | k | v | gate logits]: q and k each divided by the root mean
+        square of their WHOLE projection and multiplied by q_norm [heads * dim] / k_norm [kv_heads * dim] (None:
+        no norm), rotated (the first r dims of a head in two halves), q times head_scale[head] (float32 [heads]
+        or None); k and v stored in the pages at `slot_mapping` (negative: not stored).  All in 32-bit, one
+        rounding.  Returns q [T, heads * head_dim] in the engine's dtype (heads padded with zeros to the pages'
+        head size) and, if `gated`, sigmoid(gate logits) float32 [T, heads]."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        if width < num_heads * dim + num_kv_heads * (dim + value_dim) + (num_heads if gated else 0):
+            raise KernelError("the projected rows are too narrow")
+        weight_f32 = 0
+        for w, n, name in ((q_norm, num_heads * dim, "query norm weight"), (k_norm, num_kv_heads * dim, "key norm weight")):
+            if w is not None:
+                self._check(w, name, (torch.float32, self.dtype), (n,))
+                weight_f32 = int(w.dtype == torch.float32)
+        if q_norm is not None and k_norm is not None and q_norm.dtype != k_norm.dtype:
+            raise KernelError("the two norm weights must have one dtype")
+        if head_scale is not None:
+            self._check(head_scale, "head scale", torch.float32, (num_heads,))
+        cos = sin = None
+        rotary = 0
+        if rotation is not None:
+            cos, sin, rotary = rotation
+            if rotary <= 0 or rotary % 2 or rotary > dim:
+                raise KernelError("rotary_dim must be even and within dim")
+            self._check(cos, "rotary cos", torch.float32, (tokens, rotary // 2))
+            self._check(sin, "rotary sin", torch.float32, (tokens, rotary // 2))
+        num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+        self._check(slot_mapping, "slot mapping", torch.int32, (tokens,))
+        q = self._empty((tokens, num_heads * head_dim), self.dtype)
+        gate = self._empty((tokens, num_heads), torch.float32) if gated else None
+        self._call(
+            "mlr_qk_norm_rope_write", self._ptr(projected), width, self._ptr(q_norm), self._ptr(k_norm), weight_f32,
+            float(eps), self._ptr(head_scale), self._ptr(cos), self._ptr(sin), int(rotary), self._ptr(slot_mapping),
+            self._ptr(key_pages), self._ptr(value_pages), self._ptr(q), self._ptr(gate), self.code, tokens, num_heads,
+            num_kv_heads, dim, value_dim, head_dim, block_size, num_pages, int(bool(gated)), self._stream(),
+        )
+        return q, gate
+
+    def pool_kv_write(
+        self,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        block_table: torch.Tensor,
+        pooled_slots: torch.Tensor,
+        pooled_keys: torch.Tensor,
+        pooled_values: torch.Tensor,
+        ctx: Any,
+        *,
+        num_kv_heads: int,
+        head_dim: int,
+        block_size: int,
+        pool: int,
+    ) -> None:
+        """Every token of the step that completes a run of `pool` positions (pooled_slots[t] >= 0) stores the means
+        of the run's keys and of its values, as the token pages hold them, at that slot of the pooled pages."""
+        num_pages = self._check_pages(key_pages, value_pages, num_kv_heads, head_dim, block_size)
+        pooled_pages = self._check_pages(pooled_keys, pooled_values, num_kv_heads, head_dim, block_size)
+        tokens = pooled_slots.shape[0]
+        self._check(pooled_slots, "pooled slot mapping", torch.int32, (tokens,))
+        self._check(block_table, "block table", torch.int32, (ctx.num_entries, None))
+        self._check(ctx.token_entry, "token entries", torch.int32, (tokens,))
+        self._check(ctx.positions, "positions", torch.int32, (tokens,))
+        if pool <= 0:
+            raise KernelError("a run has at least one position")
+        self._call(
+            "mlr_pool_kv_write", self._ptr(key_pages), self._ptr(value_pages), self._ptr(block_table), block_table.shape[1],
+            num_pages, self._ptr(ctx.token_entry), self._ptr(ctx.positions), self._ptr(pooled_slots), self._ptr(pooled_keys),
+            self._ptr(pooled_values), pooled_pages, self.code, tokens, num_kv_heads, head_dim, block_size, int(pool),
+            self._stream(),
+        )
+
+    def scale_heads(
+        self,
+        attended: torch.Tensor,
+        gate: Optional[torch.Tensor],
+        *,
+        heads: int,
+        head_dim: int,
+        out_dim: int,
+        scale: float = 1.0,
+        out: Optional[torch.Tensor] = None,
+        column: int = 0,
+    ) -> torch.Tensor:
+        """The first `out_dim` dims of every head of attended [T, heads * head_dim], times gate[t, head] (float32 [T,
+        heads] or None) and `scale`: [T, heads * out_dim], or columns column .. of the wider `out`."""
+        self._check(attended, "attended heads", self.dtype, (None, heads * head_dim))
+        tokens = attended.shape[0]
+        if gate is not None:
+            self._check(gate, "head gates", torch.float32, (tokens, heads))
+        if not 0 < out_dim <= head_dim:
+            raise KernelError("out_dim must lie within head_dim")
+        out, view, row = self._columns(out, column, tokens, heads * out_dim)
+        self._call(
+            "mlr_scale_heads", self._ptr(attended), self._ptr(gate), view, row, self.code, tokens, heads, head_dim,
+            out_dim, float(scale), self._stream(),
+        )
+        return out
+
+    def gla_scan(
+        self,
+        projected: torch.Tensor,
+        state: torch.Tensor,
+        read_rows: torch.Tensor,
+        write_rows: torch.Tensor,
+        ctx: Any,
+        *,
+        heads: int,
+        head_dim: int,
+        value_dim: int,
+        decay_weight: torch.Tensor,
+        decay_bias: Optional[torch.Tensor],
+        low_offset: int,
+        tau: float,
+        q_scale: float,
+    ) -> torch.Tensor:
+        """Linear attention with a decay per key channel and token, every entry's tokens in order: S = diag(a_t) S +
+        k_t v_t^T, o_t = S^T (q_t * q_scale) per head, a_t = sigmoid(W2 low_t + bias)^(1 / tau) with low_t the columns
+        low_offset .. low_offset + rank of `projected` (float32 [T, q | k | v | ...]) and W2 = decay_weight [heads *
+        head_dim, rank].  State rows as for `retention_scan`.  Everything in 32-bit.  Returns o, float32 [T, heads *
+        value_dim]."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        entries = ctx.num_entries
+        self._check(decay_weight, "decay weight", (torch.float32, self.dtype), (heads * head_dim, None))
+        rank = decay_weight.shape[1]
+        if decay_bias is not None:
+            self._check(decay_bias, "decay bias", (torch.float32, self.dtype), (heads * head_dim,))
+        if low_offset < 0 or low_offset + rank > width or 2 * heads * head_dim + heads * value_dim > width:
+            raise KernelError("the projected rows do not hold q, k, v and the decay's inputs")
+        self._check(state, "recurrent state", torch.float32, (None, heads, head_dim, value_dim))
+        self._check(read_rows, "state rows to read", torch.int32, (entries,))
+        self._check(write_rows, "state rows to write", torch.int32, (entries,))
+        self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
+        self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
+        out = self._empty((tokens, heads * value_dim), torch.float32)
+        decay = self._empty((tokens, heads * head_dim), torch.float32)
+        self._call(
+            "mlr_gla_scan", self._ptr(projected), width, int(low_offset), rank, self._ptr(decay_weight),
+            self._ptr(decay_bias), int(decay_weight.dtype == torch.float32),
+            int(decay_bias is not None and decay_bias.dtype == torch.float32), float(tau), self._ptr(decay),
+            self._ptr(state), state.shape[0], self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.cu_q),
+            self._ptr(ctx.q_starts), float(q_scale), self._ptr(out), entries, heads, head_dim, value_dim, tokens,
+            self._stream(),
         )
         return out
 

@@ -23,6 +23,9 @@ class Architecture:
     name: str
     config_class: Type[ModelConfig]
     build_spec: Callable[[ModelConfig], ModelSpec]
+    # (config, {tensor name: stored shape}) -> config: for an architecture some of whose sizes no
+    # config.json key gives, only a stored tensor's shape; None when config.json says everything
+    with_shapes: Any = None
 
 
 ARCHITECTURES: dict[str, Architecture] = {}
@@ -34,10 +37,11 @@ def register_architecture(
     build_spec: Callable[[Any], ModelSpec],
     *,
     replace: bool = False,
+    with_shapes: Any = None,
 ) -> Architecture:
     if name in ARCHITECTURES and not replace:
         raise ValueError(f"architecture {name!r} is already registered")
-    arch = Architecture(name, config_class, build_spec)
+    arch = Architecture(name, config_class, build_spec, with_shapes)
     ARCHITECTURES[name] = arch
     return arch
 
@@ -72,7 +76,25 @@ def config_from_dict(data: Mapping[str, Any]) -> ModelConfig:
 
 
 def load_config(model_dir: str | Path) -> ModelConfig:
-    return config_from_dict(read_config_json(model_dir))
+    """The configuration of a model folder: config.json, completed from the shapes of the stored
+    tensors where the architecture says that some of its sizes are only there."""
+    data = read_config_json(model_dir)
+    arch = architecture_of(data)
+    config = arch.config_class.from_dict(data)
+    if arch.with_shapes is not None:
+        from ..weights.loader import checkpoint_files
+
+        try:
+            files = checkpoint_files(model_dir)
+        except FileNotFoundError:
+            return config  # a folder without weights: the sizes keep their defaults
+        try:
+            shapes = {name: tuple(e.shape) for f in files.values() for name, e in f.entries.items()}
+        finally:
+            for f in files.values():
+                f.close()
+        config = arch.with_shapes(config, shapes)
+    return config
 
 
 def build_spec(config: ModelConfig) -> ModelSpec:

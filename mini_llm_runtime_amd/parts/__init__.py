@@ -1,6 +1,9 @@
 """Parts a layer is put together from, and the model that runs them."""
 
-from . import attention, block, feed_forward, latent_attention, norm, position, retention, token_input  # noqa: F401  (register the built-in kinds)
+from . import (  # noqa: F401  (register the built-in kinds)
+    attention, block, feed_forward, gated_linear_attention, latent_attention, norm, pooled_attention, position, retention,
+    short_conv, side_by_side, token_input,
+)
 from .base import Block, FeedForward, Mixer, Norm, Part, PositionEncoding
 from .context import KVView, StateView, StepContext
 from .model import DecoderModel

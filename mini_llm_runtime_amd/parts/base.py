@@ -39,6 +39,10 @@ class Part:
         for name, tensor in params.items():
             setattr(self, name, tensor)
 
+    def bound(self) -> None:
+        """Called once every part of the model has received its parameters, nested parts before the
+        parts that hold them: for what a part makes of its children's tensors."""
+
     def children(self) -> dict[str, "Part"]:
         """Parts nested inside this one (their parameters live under `<name>.`)."""
         return {}
@@ -90,7 +94,24 @@ class Mixer(Part):
         return None
 
     def forward(self, ctx: StepContext, h: torch.Tensor, site: int) -> torch.Tensor:
-        """h: normed activations [T, H] in the engine's dtype; returns [T, H]."""
+        """h: normed activations [T, H] in the engine's dtype; returns [T, H].  `site` is what
+        `ctx.cache` takes: the execution site's index, or the path of this mixer's member when the
+        site keeps several caches."""
+        raise NotImplementedError
+
+    # A mixer whose result is a product `activations @ o_weight^T` may leave that product to a part
+    # that holds it beside others: it then says `open_output = True`, gives the width of its
+    # activations and writes them, times `scale`, into columns column .. of a wider tensor that the
+    # holder multiplies with all its members' output matrices side by side, in one product.
+    open_output = False
+
+    @property
+    def out_width(self) -> int:
+        raise NotImplementedError
+
+    def activations(
+        self, ctx: StepContext, h: torch.Tensor, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0
+    ) -> None:
         raise NotImplementedError
 
 
@@ -101,6 +122,12 @@ class FeedForward(Part):
 
 class Block(Part):
     """An arrangement of a mixer, a feed-forward and norms around the residual stream."""
+
+    def cache_spec(self) -> Any:
+        """What an execution site of this layer keeps in the cache: the mixer's needs, unless the
+        arrangement holds more parts with a cache of their own (it then returns a `CompositeSpec`
+        and hands every part its member of the site's view)."""
+        return self.mixer.cache_spec()
 
     def forward(
         self, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor], site: int

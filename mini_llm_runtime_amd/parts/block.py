@@ -8,7 +8,8 @@ import torch
 
 from .base import Block, FeedForward, Mixer, Norm, Part
 from ..kernels.pending import NormedDelta
-from .context import StepContext
+from ..cache.spec import CompositeSpec
+from .context import StepContext, site_member
 from .registry import register_part
 
 
@@ -120,6 +121,68 @@ class SandwichNormBlock(Block):
             fed = self.token_input.forward(ctx, stream)
             owed = NormedDelta(fed, self.token_input.norm_weight, self.token_input.norm_eps)
         return x, owed
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Block):
+    """One norm, both sublayers read it, both results enter the stream together:
+
+        h = norm_input(x);   x += mixer(filter(h)) + feed_forward(h)
+
+    `mixer_filter` (optional): a part the normed activations pass on their way into the mixer only, e.g. a
+    short convolution over time with carried inputs; the feed-forward reads h as it is.  A layer may have no
+    feed-forward.  The mixer's result is added to the 32-bit stream by a kernel of its own; the
+    feed-forward's is handed to the next block un-added, like every block's last output.  What the filter
+    carries from step to step is a member of the site's cache beside the mixer's.
+    """
+
+    replayable = True
+
+    def __init__(
+        self,
+        mixer: Mixer,
+        feed_forward: Optional[FeedForward],
+        norms: Mapping[str, Norm],
+        mixer_filter: Optional[Part] = None,
+    ) -> None:
+        if "input" not in norms:
+            raise ValueError("parallel block needs the norm 'input'")
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_filter = mixer_filter
+        self.norm_input = norms["input"]
+        filter_spec = mixer_filter.cache_spec() if mixer_filter is not None and hasattr(mixer_filter, "cache_spec") else None
+        self._filter_keeps = filter_spec is not None
+
+    def children(self) -> dict[str, Part]:
+        parts: dict[str, Part] = {"mixer": self.mixer, "norm_input": self.norm_input}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+        if self.mixer_filter is not None:
+            parts["mixer_filter"] = self.mixer_filter
+        return parts
+
+    def cache_spec(self):
+        own = self.mixer.cache_spec()
+        if not self._filter_keeps:
+            return own
+        members = {"filter": self.mixer_filter.cache_spec()}
+        if own is not None:
+            members["mixer"] = own
+        return CompositeSpec(members)
+
+    def forward(
+        self, ctx: StepContext, x: torch.Tensor, delta, site: int
+    ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        h = self.norm_input.forward(ctx, x, delta)
+        m = h
+        if self.mixer_filter is not None:
+            m = self.mixer_filter.forward(ctx, h, site_member(site, "filter") if self._filter_keeps else site)
+        mixed = self.mixer.forward(ctx, m, site_member(site, "mixer") if self._filter_keeps else site)
+        if self.feed_forward is None:
+            return x, mixed
+        ctx.ops.add_(x, mixed)
+        return x, self.feed_forward.forward(ctx, h)
 
 
 def _norm(norm: Norm, consumer: Part, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor]):

@@ -14,6 +14,11 @@ import torch
 from ..cache.views import KVView, StateView  # noqa: F401  (part of this module's surface)
 
 
+def site_member(site: Any, name: str) -> tuple:
+    """The path of member `name` of the composite cache that `site` (an index or a path) names."""
+    return (*site, name) if isinstance(site, tuple) else (site, name)
+
+
 @dataclass(frozen=True)
 class PlanInput:
     """What a mixer may look at when it plans its kernels for a step: the new tokens and the
@@ -70,15 +75,22 @@ class StepContext:
         the plan's sizes and, as device tensors, its arrays."""
         return self.plans.get(key)
 
-    def cache(self, site: int) -> Any:
-        """The view of the cache that execution site `site` uses in this step, as its spec made it."""
+    def cache(self, site: Any) -> Any:
+        """The view of the cache that execution site `site` uses in this step, as its spec made it.
+        `site` is the site's index, or a path (index, member name, ...) into a site whose spec is a
+        composite: a part that holds other parts hands each the path of its member."""
+        if isinstance(site, tuple):
+            view = self.site_views[site[0]]
+            for name in site[1:]:
+                view = view[name]
+            return view
         return self.site_views[site]
 
-    def kv(self, site: int) -> KVView:
-        return self.site_views[site]
+    def kv(self, site: Any) -> KVView:
+        return self.cache(site)
 
-    def state(self, site: int) -> StateView:
-        return self.site_views[site]
+    def state(self, site: Any) -> StateView:
+        return self.cache(site)
 
     # the views by the names they had when there were two kinds
     @property

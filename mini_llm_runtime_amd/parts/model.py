@@ -24,6 +24,8 @@ def _build_layer(spec: LayerSpec) -> Block:
     extra = {}
     if spec.token_input is not None:  # only arrangements that take one are handed one
         extra["token_input"] = build_part("token_input", spec.token_input)
+    if spec.mixer_filter is not None:
+        extra["mixer_filter"] = build_part("input_filter", spec.mixer_filter)
     return build_part("block", PartSpec(spec.block), mixer=mixer, feed_forward=feed_forward, norms=norms, **extra)
 
 
@@ -52,7 +54,7 @@ class DecoderModel:
         for site, entry in enumerate(spec.order):
             if not 0 <= entry.layer < len(self.layers):
                 raise ValueError(f"order entry {site} names layer {entry.layer}, the model has {len(self.layers)}")
-            own = self.layers[entry.layer].mixer.cache_spec()
+            own = self.layers[entry.layer].cache_spec()
             if entry.reads_cache_of is not None:
                 src = entry.reads_cache_of
                 if not 0 <= src < site or spec.order[src].reads_cache_of is not None:
@@ -123,6 +125,8 @@ class DecoderModel:
         for path, part in self.named_parts():
             own = {name: params[f"{path}.{name}"] for name in part.param_specs()}
             part.bind(own, dtype=dtype, device=self.device)
+        for _, part in reversed(list(self.named_parts())):  # children before the parts that hold them
+            part.bound()
 
     def weight_bytes(self) -> int:
         seen: dict[int, int] = {}

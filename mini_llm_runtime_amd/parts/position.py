@@ -30,7 +30,14 @@ class RotaryEmbedding(PositionEncoding):
     max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), r - 1) and ramp_j = clamp((j - lo) / max(hi -
     lo, 0.001), 0, 1), pair j turns at f_j / factor * ramp_j + f_j * (1 - ramp_j): fast pairs keep
     their frequency, slow ones are stretched by `factor`.  Cosines and sines are then multiplied by
-    0.1 ln(factor) + 1.
+    0.1 ln(factor) + 1.  A scaling that gives `factor` alone is the linear one: every pair turns at f_j /
+    factor, amplitudes stay 1.
+
+    interleaved: the checkpoint pairs dim 2j with dim 2j + 1 (instead of j with j + r/2).  The kernels
+    rotate halves; a dot product of a query and a key does not care in which order both list their
+    dims, so a mixer that projects q and k reorders the rows of both projections once, when its weights
+    are bound, by `half_split_order()` (pair j's first members to the front half, its second members
+    behind them), and everything after that is the half-split rotation.
     """
 
     replayable = True
@@ -41,7 +48,9 @@ class RotaryEmbedding(PositionEncoding):
         theta: float,
         rotary_dim: Optional[int] = None,
         scaling: Optional[Mapping[str, float]] = None,
+        interleaved: bool = False,
     ) -> None:
+        self.interleaved = bool(interleaved)
         rotary_dim = head_dim if rotary_dim is None else int(rotary_dim)
         if rotary_dim <= 0 or rotary_dim % 2 or rotary_dim > head_dim:
             raise ValueError("rotary_dim must be even and within head_dim")
@@ -54,7 +63,13 @@ class RotaryEmbedding(PositionEncoding):
         self._inv_freq_host = 1.0 / (self.theta**exponents)
         self.amplitude = 1.0
         self.scaling = None
-        if scaling is not None:
+        if scaling is not None and "original" not in scaling:
+            factor = float(scaling["factor"])
+            if not factor > 0:
+                raise ValueError("the factor of a rotary scaling must be > 0")
+            self.scaling = (factor,)
+            self._inv_freq_host = self._inv_freq_host / factor
+        elif scaling is not None:
             factor, original = float(scaling["factor"]), float(scaling["original"])
             fast, slow = float(scaling["fast"]), float(scaling["slow"])
             if not (factor > 0 and original > 0 and fast > 0 and slow > 0):
@@ -73,6 +88,14 @@ class RotaryEmbedding(PositionEncoding):
 
     def bind(self, params: Mapping[str, torch.Tensor], *, dtype: torch.dtype, device: torch.device) -> None:
         self.inv_freq = torch.from_numpy(self._inv_freq_host).to(device)
+
+    def half_split_order(self) -> list[int]:
+        """For every dim of a head in the order the kernels want, the dim of the checkpoint's order
+        that goes there (the identity unless `interleaved`)."""
+        r = self.rotary_dim
+        if not self.interleaved:
+            return list(range(self.head_dim))
+        return list(range(0, r, 2)) + list(range(1, r, 2)) + list(range(r, self.head_dim))
 
     def rotation(self, ctx: StepContext):
         key = ("rotary", self.rotary_dim, self.theta, self.scaling)

@@ -9,7 +9,7 @@ from typing import Any, Callable
 
 from .spec import PartSpec
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "token_input")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "token_input", "input_filter")
 
 _REGISTRY: dict[str, dict[str, Callable[..., Any]]] = {c: {} for c in CATEGORIES}
 

@@ -39,13 +39,16 @@ class LayerSpec:
     """One layer: an arrangement (`block`) of a mixer, a feed-forward (None: the layer has
     none, if its arrangement allows that) and norms.  `token_input`: a part that feeds something
     of the token itself into the stream at this layer (None: the layer has none); only
-    arrangements that know what to do with one take it."""
+    arrangements that know what to do with one take it.  `mixer_filter`: a part that the normed
+    activations pass on their way into the mixer (and only there), e.g. a short convolution over
+    time; likewise only for arrangements that take one."""
 
     block: str
     mixer: PartSpec
     feed_forward: Optional[PartSpec]
     norms: Mapping[str, PartSpec]
     token_input: Optional[PartSpec] = None
+    mixer_filter: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)

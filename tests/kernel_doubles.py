@@ -63,7 +63,8 @@ class TorchOps:
         return (weight.float() * (x * torch.rsqrt(variance + eps))).to(self.dtype)
 
     def add_(self, x, delta):
-        x += delta.float()
+        delta = self.settle(delta)
+        x += self._sum(delta) if delta.dim() == x.dim() + 1 else delta.float()
 
     def scale_softcap_(self, x, scale=1.0, cap=None):
         x *= scale
@@ -198,13 +199,130 @@ class TorchOps:
             state[int(write_rows[r])] = s
         return out.view(tokens, heads * value_dim)
 
-    def retention_gate(self, retained, projected, *, heads, value_dim, gate_offset, eps):
+    def retention_gate(
+        self, retained, projected, *, heads, value_dim, gate_offset, eps, norm_weight=None, scale=1.0, out=None, column=0
+    ):
         self._count("retention_gate")
         tokens = retained.shape[0]
         o = retained.float().view(tokens, heads, value_dim)
         o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        if norm_weight is not None:
+            o = o * norm_weight.float()
         z = projected[:, gate_offset : gate_offset + heads * value_dim].float()
-        return (o.reshape(tokens, heads * value_dim) * (z * torch.sigmoid(z))).to(self.dtype)
+        y = (o.reshape(tokens, heads * value_dim) * (z * torch.sigmoid(z)) * scale).to(self.dtype)
+        if out is None:
+            return y
+        out[:, column : column + heads * value_dim] = y
+        return out
+
+    # parts that run side by side ---------------------------------------------------------------
+    def short_conv(self, h, weight, state, read_rows, write_rows, ctx, *, add_input=True):
+        self._count("short_conv")
+        taps = weight.shape[1]
+        carried = taps - 1
+        w = weight.float()
+        out = torch.zeros_like(h, dtype=torch.float32)
+        for r in range(ctx.num_entries):
+            a, b = int(ctx.cu_q[r]), int(ctx.cu_q[r + 1])
+            before = torch.zeros(carried, h.shape[1])
+            if carried and int(ctx.q_starts[r]) > 0:
+                before = state[int(read_rows[r])].float().clone()
+            seq = torch.cat([before, h[a:b].float()])
+            for j in range(taps):
+                out[a:b] += w[:, j] * seq[j : j + (b - a)]
+            if add_input:
+                out[a:b] += h[a:b].float()
+            if carried:
+                state[int(write_rows[r])] = seq[seq.shape[0] - carried :]
+        return out.to(self.dtype)
+
+    def qk_norm_rope_write(
+        self, projected, q_norm, k_norm, eps, head_scale, rotation, slot_mapping, key_pages, value_pages, *, num_heads,
+        num_kv_heads, dim, value_dim, head_dim, block_size, gated=False,
+    ):
+        self._count("qk_norm_rope_write")
+        tokens = projected.shape[0]
+        p = projected.float()
+        qs, ks, vs = num_heads * dim, num_kv_heads * dim, num_kv_heads * value_dim
+        q, k, v = p[:, :qs], p[:, qs : qs + ks], p[:, qs + ks : qs + ks + vs]
+        if q_norm is not None:
+            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()
+        if k_norm is not None:
+            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.float()
+        q = self._rotate(q.reshape(tokens, num_heads, dim), rotation)
+        k = self._rotate(k.reshape(tokens, num_kv_heads, dim), rotation)
+        if head_scale is not None:
+            q = q * head_scale.float()[None, :, None]
+        q_out = torch.zeros(tokens, num_heads, head_dim)
+        q_out[..., :dim] = q
+        k_out = torch.zeros(tokens, num_kv_heads, head_dim)
+        k_out[..., :dim] = k
+        v_out = torch.zeros(tokens, num_kv_heads, head_dim)
+        v_out[..., :value_dim] = v.reshape(tokens, num_kv_heads, value_dim)
+        slots = slot_mapping.long()
+        ok = slots >= 0
+        page, off = slots[ok] // block_size, slots[ok] % block_size
+        key_pages[page, :, off, :] = k_out[ok].to(key_pages.dtype)
+        value_pages[page, :, :, off] = v_out[ok].to(value_pages.dtype)
+        gate = torch.sigmoid(p[:, qs + ks + vs : qs + ks + vs + num_heads]) if gated else None
+        return q_out.reshape(tokens, num_heads * head_dim).to(self.dtype), gate
+
+    def pool_kv_write(
+        self, key_pages, value_pages, block_table, pooled_slots, pooled_keys, pooled_values, ctx, *, num_kv_heads, head_dim,
+        block_size, pool,
+    ):
+        self._count("pool_kv_write")
+        table = block_table.long()
+        for t in range(pooled_slots.shape[0]):
+            slot = int(pooled_slots[t])
+            if slot < 0:
+                continue
+            p = int(ctx.positions[t])
+            idx = torch.arange(p - pool + 1, p + 1)
+            page = table[int(ctx.token_entry[t]), idx // block_size]
+            assert (page >= 0).all(), "a run is pooled from pages that are not there"
+            k = key_pages[page, :, idx % block_size, :].float().mean(0)  # [Hkv, d]
+            v = value_pages[page, :, :, idx % block_size].float().mean(0)
+            pooled_keys[slot // block_size, :, slot % block_size, :] = k.to(pooled_keys.dtype)
+            pooled_values[slot // block_size, :, :, slot % block_size] = v.to(pooled_values.dtype)
+
+    def scale_heads(self, attended, gate, *, heads, head_dim, out_dim, scale=1.0, out=None, column=0):
+        self._count("scale_heads")
+        tokens = attended.shape[0]
+        y = attended.float().view(tokens, heads, head_dim)[..., :out_dim] * scale
+        if gate is not None:
+            y = y * gate.float()[:, :, None]
+        y = y.reshape(tokens, heads * out_dim).to(self.dtype)
+        if out is None:
+            return y
+        out[:, column : column + heads * out_dim] = y
+        return out
+
+    def gla_scan(
+        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, decay_weight, decay_bias,
+        low_offset, tau, q_scale,
+    ):
+        self._count("gla_scan")
+        tokens = projected.shape[0]
+        p = projected.float()
+        qk = heads * head_dim
+        q = p[:, :qk].view(tokens, heads, head_dim) * q_scale
+        k = p[:, qk : 2 * qk].view(tokens, heads, head_dim)
+        v = p[:, 2 * qk : 2 * qk + heads * value_dim].view(tokens, heads, value_dim)
+        rank = decay_weight.shape[1]
+        z = p[:, low_offset : low_offset + rank] @ decay_weight.float().T
+        if decay_bias is not None:
+            z = z + decay_bias.float()
+        alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(tokens, heads, head_dim)
+        out = torch.zeros(tokens, heads, value_dim, dtype=torch.float32)
+        for r in range(ctx.num_entries):
+            a, b = int(ctx.cu_q[r]), int(ctx.cu_q[r + 1])
+            s = state[int(read_rows[r])].float().clone() if int(ctx.q_starts[r]) > 0 else torch.zeros_like(state[0])
+            for t in range(a, b):
+                s = alpha[t][:, :, None] * s + k[t][:, :, None] * v[t][:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", s, q[t])
+            state[int(write_rows[r])] = s
+        return out.view(tokens, heads * value_dim)
 
     def rope_kv_write(
         self, qkv, rotation, slot_mapping, key_pages, value_pages, *, num_heads, num_kv_heads, head_dim, block_size, write=True
@@ -241,7 +359,7 @@ class TorchOps:
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
-        defer_merge=False, plan=None, chunk=None, sinks=None,
+        defer_merge=False, plan=None, chunk=None, sinks=None, pooled=None,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]
@@ -260,6 +378,13 @@ class TorchOps:
             assert (page >= 0).all(), "attention would read a page that is not there"
             k = key_pages[page, :, idx % block_size, :].float()  # [n, Hkv, d]
             v = value_pages[page, :, :, idx % block_size].float()
+            if pooled is not None and p - window >= 0:  # the runs that end at or before p - window, through their means
+                pk, pv, ptable, pool = pooled
+                runs = torch.arange((p - window + 1) // pool)
+                ppage = ptable.long()[r, runs // block_size]
+                assert (ppage >= 0).all(), "attention would read a pooled page that is not there"
+                k = torch.cat([pk[ppage, :, runs % block_size, :].float(), k])
+                v = torch.cat([pv[ppage, :, :, runs % block_size].float(), v])
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)
             s = torch.einsum("hd,nhd->hn", q[t], k) * scale
