@@ -97,12 +97,18 @@ def vobisun_spec(config: VobisunConfig) -> ModelSpec:
         if layer.ff is not None:
             feed_forward = PartSpec("swiglu", {"hidden_size": width, "intermediate_size": layer.ff})
             ff = dst + "feed_forward."
-            rules += [
+            if layer.ff % 2 == 0:
                 # gate and up rows woven in pairs: the product's epilogue then holds a gate sum beside its up sum
-                WeightRule(src + "mlp.gate", ff + "gate_up_weight", 0, layer.ff, block=2, period=4),
-                WeightRule(src + "mlp.up", ff + "gate_up_weight", 2, layer.ff, block=2, period=4),
-                WeightRule(src + "mlp.down", ff + "down_weight"),
-            ]
+                rules += [
+                    WeightRule(src + "mlp.gate", ff + "gate_up_weight", 0, layer.ff, block=2, period=4),
+                    WeightRule(src + "mlp.up", ff + "gate_up_weight", 2, layer.ff, block=2, period=4),
+                ]
+            else:  # an odd size cannot be woven: the gating runs behind the product
+                rules += [
+                    WeightRule(src + "mlp.gate", ff + "gate_up_weight", 0, layer.ff),
+                    WeightRule(src + "mlp.up", ff + "gate_up_weight", layer.ff, layer.ff),
+                ]
+            rules.append(WeightRule(src + "mlp.down", ff + "down_weight"))
         layers.append(
             LayerSpec(
                 block="parallel", mixer=mixer, feed_forward=feed_forward, norms={"input": norm},

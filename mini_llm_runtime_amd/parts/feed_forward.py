@@ -19,17 +19,20 @@ class SwiGLU(FeedForward):
     Formula: src/mini_llm_runtime/qwen_model_runner.py:215-217.  Gate and up are one
     matrix product over a matrix that holds the rows of Wgate and Wup woven in pairs
     (gate 0, gate 1, up 0, up 1, gate 2, ...; made by the weight rules), and
-    silu(gate) * up is that product's epilogue.
+    silu(gate) * up is that product's epilogue.  An odd intermediate size cannot be woven in
+    pairs (`woven` is False): its rows are [Wgate ; Wup] and the gating is a kernel of its own
+    behind the product.
     """
 
     replayable = True
     takes_pending_norm = True  # `h` goes to the gate/up product only
 
     def __init__(self, hidden_size: int, intermediate_size: int) -> None:
-        if hidden_size <= 0 or intermediate_size <= 0 or intermediate_size % 2:
-            raise ValueError("SwiGLU sizes must be > 0 and the intermediate size even")
+        if hidden_size <= 0 or intermediate_size <= 0:
+            raise ValueError("SwiGLU sizes must be > 0")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        self.woven = self.intermediate_size % 2 == 0
         self.gate_up_weight: Optional[torch.Tensor] = None
         self.down_weight: Optional[torch.Tensor] = None
 
@@ -41,7 +44,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
-        hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
+        if self.woven:
+            hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
+        else:
+            hidden = ops.silu_mul(ops.linear(h, self.gate_up_weight, None))
         return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta
 
 

@@ -76,11 +76,26 @@ def test_a_head_size_no_kernel_runs_is_refused_when_the_model_is_built():
         build_model(too_wide)
 
 
-def test_an_odd_intermediate_size_is_refused_when_the_model_is_built():
+def test_an_odd_intermediate_size_runs_unwoven(tmp_path):
     """Gate and up rows are woven in pairs for the SwiGLU epilogue: an odd number of them has no such
-    layout, and the feed-forward says so instead of computing something else."""
-    with pytest.raises(ValueError, match="intermediate size even"):
-        build_model(Qwen2Config.from_dict({**TINY_A, "intermediate_size": 129}))
+    layout, so they are stored [gate ; up] and the gating runs behind the product."""
+    import json
+
+    import plain_qwen2 as plain
+    from kernel_doubles import TorchOps
+    from helpers import StepEntry, make_runner, random_tokens
+
+    config = Qwen2Config.from_dict({**TINY_A, "intermediate_size": 129})
+    assert build_model(config).layers[0].feed_forward.woven is False
+    import mini_llm_runtime_amd as mlr
+
+    folder = mlr.write_random_model(config, tmp_path / "odd", seed=3, storage_dtype="bfloat16")
+    cfg, weights = read_weights(folder)
+    toks = random_tokens(9, config.vocab_size, 2)
+    _, _, cache, runner = make_runner(folder, TorchOps(torch.float32, "cpu"), block_size=8, num_blocks=4, max_requests=1)
+    cache.create_request("a")
+    got = runner.step([StepEntry.of("a", toks, list(range(9)))]).logits.double()
+    torch.testing.assert_close(got, plain.forward(toks, weights, cfg).double(), rtol=1e-4, atol=1e-4)
 
 
 def test_random_model_is_seeded_and_loads(tmp_path):

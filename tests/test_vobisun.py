@@ -1,0 +1,691 @@
+"""The Vobisun decoder in the engine against the plain implementation (`plain_vobisun.py`).
+
+Each mechanism alone (the short convolution with carried inputs, the recurrence with a decay per key channel
+and its state rows, one-layer models in which only one half of the mixer counts), keys placed at every edge of
+the window and of the pooled blocks so that one score stands out, a sink that decides, a state that never
+forgets, then whole models under every way of cutting and batching over poisoned pages and reused slots,
+replays against unrecorded steps, and greedy generation through the engine, the command line and the replay
+program.  The tests make their own small configurations and weights; sizes differ from layer to layer, also
+where a model could make them equal (heads and key/value heads, key and value sizes, window and pooled block,
+rotated and unrotated dims, a factor of 1, one tap).
+
+`double` cases run everything above the kernels on the CPU stand-in; `hip` cases run the HIP kernels
+(`-m gpu`) in float32 and bfloat16.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+from pathlib import Path
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import mini_llm_runtime_amd.models  # noqa: F401
+import plain_vobisun as plain
+import schedules
+from helpers import make_runner, random_tokens
+from kernel_doubles import TorchOps
+from mini_llm_runtime_amd.config import ConfigError
+from mini_llm_runtime_amd.config.vobisun import VobisunConfig
+from mini_llm_runtime_amd.engine import ContinuousBatchEngine
+from mini_llm_runtime_amd.models import build_model, config_from_dict
+from mini_llm_runtime_amd.weights import save_state_dict
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+# ---- configurations -----------------------------------------------------------------------------------
+
+def _left(heads, kv_heads, dim, vdim, window, pool, rot_dims, factor=None, scale=0.2, base=10000.0):
+    rot = {"base": base, "dims": rot_dims}
+    if factor is not None:
+        rot["scaling"] = {"factor": factor}
+    return {
+        "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
+        "mask": {"size": window, "pool": pool}, "rot": rot,
+    }
+
+
+def _right(heads, dim, vdim, tau):
+    return {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau}
+
+
+def _layer(left, right, ff, left_scale=1.0, right_scale=1.0):
+    return {
+        "type": "parallel",
+        "mixer": {"left": left, "left_scale": left_scale, "right": right, "right_scale": right_scale},
+        "mlp": None if ff is None else {"kind": "dense", "ff": ff},
+    }
+
+
+def _model(vocab, width, eps, scale, taps, layers, loop=None):
+    cfg = {
+        "architecture": "Vobisun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "embedding": {"scale": scale},
+        "canon": {"taps": taps}, "layers": layers,
+    }
+    if loop is not None:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+CONFIGS = {
+    # two key/value heads for four query heads, values wider than keys, a window that is no multiple of the
+    # pooled block or the page, a partial stretched rotation; a second layer with other sizes everywhere, no
+    # feed-forward, a full unstretched rotation; the first layer runs twice
+    "A": _model(300, 64, 1e-6, 4.0, 4, [
+        _layer(_left(4, 2, 16, 24, 10, 4, 8, 2.0), _right(2, 16, 32, 8.0), 96, 0.7, 1.3),
+        _layer(_left(2, 1, 32, 16, 7, 3, 32), _right(3, 8, 16, 2.0), None, 1.0, 0.5),
+    ], loop=(0, 1, 2)),
+    # sizes that the matrix-core kernels refuse: a width of 72, heads of 10 dims of which 4 turn, values of 12,
+    # as many key/value heads as heads, a pooled block longer than the window, two taps, an odd vocabulary
+    "B": _model(257, 72, 1e-5, 1.0, 2, [
+        _layer(_left(3, 3, 10, 12, 5, 8, 4, None, 0.3, 777.0), _right(3, 20, 12, 1.0), 52, 1.1, -0.9),
+        _layer(_left(2, 1, 12, 6, 9, 2, 6, 1.5, 0.25), _right(1, 24, 40, 3.0), 44, 0.5, 1.0),
+    ]),
+    # matrix-core sizes; three layers of which the last two run three times
+    "C": _model(512, 128, 1e-5, 8.0, 3, [
+        _layer(_left(8, 2, 32, 32, 48, 16, 32, 8.0, 0.18, 1e6), _right(4, 64, 32, 16.0), 192, 1.2, 0.8),
+        _layer(_left(4, 4, 64, 48, 33, 8, 16, None, 0.12), _right(2, 32, 64, 4.0), 160),
+        _layer(_left(16, 1, 16, 16, 64, 32, 8, 3.0, 0.25), _right(8, 16, 16, 32.0), None, 0.9, 1.1),
+    ], loop=(1, 3, 3)),
+    # long requests: hundreds of keys in the window (the decode kernel's partitions and their merge), dozens of
+    # pooled blocks, states that carry over hundreds of tokens
+    "D": _model(200, 128, 1e-5, 6.0, 3, [
+        _layer(_left(4, 1, 32, 48, 300, 8, 16, 4.0, 0.2), _right(2, 64, 64, 64.0), 96),
+        _layer(_left(2, 2, 64, 32, 40, 5, 64, None, 0.15), _right(4, 32, 16, 8.0), None),
+    ]),
+    # values that could hide a fault by being 1: one tap (no carried inputs), a window of one token, pooled
+    # blocks of one token (every older token is its own block), one head everywhere, a loop that runs once
+    "E": _model(96, 48, 1e-6, 1.0, 1, [
+        _layer(_left(1, 1, 16, 16, 1, 1, 2, 1.0, 0.3), _right(1, 16, 16, 1.0), 40),
+        _layer(_left(2, 2, 8, 8, 3, 1, 8, None, 0.4), _right(2, 8, 8, 5.0), None),
+    ], loop=(0, 2, 1)),
+    # one half of the mixer at a time: what it does is not blurred by the other
+    "L": _model(128, 64, 1e-6, 3.0, 3, [_layer(_left(4, 2, 16, 32, 12, 4, 12, 2.0, 0.3), _right(1, 8, 8, 2.0), None, 1.0, 0.0)]),
+    "R": _model(128, 64, 1e-6, 3.0, 3, [_layer(_left(1, 1, 8, 8, 4, 2, 4), _right(2, 16, 32, 6.0), None, 0.0, 1.0)]),
+}
+# what the decay's two products pass through (the stored tensor's shape says it, no key of the configuration)
+RANKS = {"A": (5, 16), "B": (7, 3), "C": (16, 8, 24), "D": (16, 12), "E": (1, 4), "L": (4,), "R": (6,)}
+BLOCK = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 4, "L": 8, "R": 4}
+LENGTHS = {
+    "A": (1, 9, 50, 83, 37, 64), "B": (2, 19, 35, 66, 45), "C": (5, 17, 140, 70, 97), "D": (660, 341),
+    "E": (1, 2, 30, 21), "L": (1, 24, 75, 41, 130), "R": (1, 24, 75, 41, 130),
+}
+
+
+def make_weights(cfg: dict, seed: int, ranks=None) -> dict[str, torch.Tensor]:
+    """bfloat16 tensors by the design's checkpoint names; queries and keys large enough for peaked attention,
+    sinks that take a visible share, decays spread between forgetting quickly and hardly at all."""
+    g = torch.Generator().manual_seed(seed)
+    width = cfg["width"]
+
+    def normal(*shape, std, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    w = {
+        "embed": normal(cfg["vocab"], width, std=1.0 / cfg["embedding"]["scale"]),
+        "final.norm": normal(width, std=0.2, mean=1.0),
+        "head": normal(cfg["vocab"], width, std=1.0 / math.sqrt(width)),
+    }
+    for i, layer in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        a, b = layer["mixer"]["left"], layer["mixer"]["right"]
+        rank = 16 if ranks is None else ranks[i]
+        w[p + "norm1"] = normal(width, std=0.2, mean=1.0)
+        w[p + "canon1"] = normal(width, cfg["canon"]["taps"], std=0.4)
+        q, k, v = a["heads"] * a["dim"], a["kv_heads"] * a["dim"], a["kv_heads"] * a["vdim"]
+        lp = p + "mix.left."
+        w[lp + "q"] = normal(q, width, std=1.0 / math.sqrt(width))
+        w[lp + "k"] = normal(k, width, std=1.0 / math.sqrt(width))
+        w[lp + "v"] = normal(v, width, std=1.0 / math.sqrt(width))
+        w[lp + "q.b"], w[lp + "k.b"], w[lp + "v.b"] = normal(q, std=0.3), normal(k, std=0.3), normal(v, std=0.3)
+        w[lp + "q.norm"], w[lp + "k.norm"] = normal(q, std=0.3, mean=2.0), normal(k, std=0.3, mean=2.0)
+        w[lp + "temp"] = normal(a["heads"], std=0.3, mean=1.2)
+        w[lp + "sink"] = normal(a["heads"], std=1.5, mean=1.0)
+        w[lp + "g"] = normal(a["heads"], width, std=1.5 / math.sqrt(width))
+        w[lp + "o"] = normal(width, a["heads"] * a["vdim"], std=1.0 / math.sqrt(a["heads"] * a["vdim"]))
+        rp = p + "mix.right."
+        qk, out = b["heads"] * b["dim"], b["heads"] * b["vdim"]
+        w[rp + "q"] = normal(qk, width, std=1.0 / math.sqrt(width))
+        w[rp + "k"] = normal(qk, width, std=1.0 / math.sqrt(width))
+        w[rp + "v"] = normal(out, width, std=1.0 / math.sqrt(width))
+        w[rp + "g"] = normal(out, width, std=1.5 / math.sqrt(width))
+        w[rp + "a1"] = normal(rank, width, std=1.0 / math.sqrt(width))
+        w[rp + "a2"] = normal(qk, rank, std=2.0 / math.sqrt(rank))
+        w[rp + "a2.b"] = normal(qk, std=2.0, mean=2.0)
+        w[rp + "norm"] = normal(b["vdim"], std=0.2, mean=1.0)
+        w[rp + "o"] = normal(width, out, std=1.0 / math.sqrt(out))
+        if layer["mlp"] is not None:
+            ff = layer["mlp"]["ff"]
+            w[p + "mlp.gate"] = normal(ff, width, std=1.5 / math.sqrt(width))
+            w[p + "mlp.up"] = normal(ff, width, std=1.5 / math.sqrt(width))
+            w[p + "mlp.down"] = normal(width, ff, std=1.0 / math.sqrt(ff))
+    return w
+
+
+def write_model(tmp_path, name: str, cfg: dict, weights: dict) -> Path:
+    folder = Path(tmp_path) / name
+    folder.mkdir(parents=True, exist_ok=True)
+    (folder / "config.json").write_text(json.dumps(cfg))
+    save_state_dict(folder / "model.safetensors", weights)
+    return folder
+
+
+def make_dir(tmp_path, which: str, seed: int = 3) -> tuple[Path, dict, dict]:
+    cfg = CONFIGS[which]
+    weights = make_weights(cfg, seed, RANKS[which])
+    return write_model(tmp_path, f"vobisun{which}", cfg, weights), cfg, weights
+
+
+def _ops(backend: str, dtype: torch.dtype):
+    if backend == "double":
+        return TorchOps(dtype, "cpu")
+    from mini_llm_runtime_amd.kernels.ops import HipOps
+
+    return HipOps(dtype, "cuda")
+
+
+CASES = [
+    pytest.param("double", torch.float32, id="double-f32"),
+    pytest.param("hip", torch.float32, id="hip-f32", marks=pytest.mark.gpu),
+    pytest.param("hip", torch.bfloat16, id="hip-bf16", marks=pytest.mark.gpu),
+]
+GPU_CASES = [
+    pytest.param(torch.float32, id="f32", marks=pytest.mark.gpu),
+    pytest.param(torch.bfloat16, id="bf16", marks=pytest.mark.gpu),
+]
+
+
+def _compare(got, requests, weights, cfg, dtype, f32_bound=2e-4, row_bound=6e-2, together=2.5e-2):
+    """float32: every value within 2e-4 of the logits' size.  bfloat16: all rows together within 2.5 %
+    (relative L2) and every row within 6 %, but for one in twenty that may be off by up to 20 %: where a sink
+    and one or two keys share the weight, or a gate is near zero, every rounding moves a row by percents.  A
+    wrong key, page, slot or state changes a row by half and more, and most rows."""
+    assert got, "no logits came back"
+    num = den = 0.0
+    loose = rows = 0
+    for rid, toks in requests.items():
+        ref = plain.forward(cfg, weights, toks)
+        size = float(ref.pow(2).mean().sqrt())
+        for pos in range(len(toks)):
+            row = got[(rid, pos)].double()
+            assert torch.isfinite(row).all(), f"{rid}:{pos} is not finite"
+            diff = row - ref[pos]
+            if dtype == torch.float32:
+                assert float(diff.abs().max()) < f32_bound * size, f"{rid}:{pos}: off by {float(diff.abs().max()):.3e} of {size:.3e}"
+                continue
+            rows += 1
+            rel = float(diff.pow(2).sum().sqrt() / ref[pos].pow(2).sum().sqrt())
+            if rel >= row_bound:
+                loose += 1
+                assert rel < 0.2, f"{rid}:{pos}: relative error {rel:.3e}"
+            num += float(diff.pow(2).sum())
+            den += float(ref[pos].pow(2).sum())
+    if dtype != torch.float32:
+        assert loose <= 0.05 * rows + 1, f"{loose} of {rows} rows are off by more than {row_bound}"
+        assert (num / den) ** 0.5 < together, f"relative error of all rows {(num / den) ** 0.5:.3e}"
+
+
+def _requests(which: str) -> dict[str, list[int]]:
+    vocab = CONFIGS[which]["vocab"]
+    return {f"r{i}": random_tokens(n, vocab, 50 + i) for i, n in enumerate(LENGTHS[which])}
+
+
+# ---- configuration and model --------------------------------------------------------------------------
+
+def test_config_reads_every_layer_by_itself():
+    c = config_from_dict(CONFIGS["A"])
+    assert isinstance(c, VobisunConfig)
+    assert c.layer_runs() == [0, 0, 1] and config_from_dict(CONFIGS["C"]).layer_runs() == [0, 1, 2, 1, 2, 1, 2]
+    assert config_from_dict(CONFIGS["B"]).layer_runs() == [0, 1]  # no loop at all
+    a, b = c.layers
+    assert (a.left.heads, a.left.kv_heads, a.left.dim, a.left.vdim, a.left.window, a.left.pool) == (4, 2, 16, 24, 10, 4)
+    assert a.left.rot.factor == 2.0 and b.left.rot.factor == 1.0 and a.left.rot.dims == 8
+    assert (a.left_scale, a.right_scale, a.ff, b.ff) == (0.7, 1.3, 96, None)
+    assert (b.right.heads, b.right.dim, b.right.vdim, b.right.tau) == (3, 8, 16, 2.0)
+    assert c.canon_taps == 4 and c.embedding_scale == 4.0
+    assert VobisunConfig.from_dict(c.to_dict()) == c
+    # the decay's inner size comes from the stored tensor
+    assert c.with_shapes({"l0.mix.right.a1": (5, 64)}).layers[0].right.rank == 5
+
+
+@pytest.mark.parametrize(
+    "change",
+    [
+        lambda c: c["layers"][0]["mixer"]["left"].pop("vdim"),
+        lambda c: c["layers"][0]["mixer"]["left"]["mask"].pop("pool"),
+        lambda c: c["layers"][0].update(type="serial"),
+        lambda c: c["layers"][0]["mixer"]["left"].update(kv_heads=3),  # four heads on three key/value heads
+        lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=18),  # more than a head has
+        lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=7),
+        lambda c: c["layers"][0]["mixer"].pop("right_scale"),
+        lambda c: c["layers"][0]["mlp"].update(kind="moe"),
+        lambda c: c["loop"].update(stop=3),  # beyond the last layer
+        lambda c: c["loop"].update(times=0),
+        lambda c: c.pop("canon"),
+        lambda c: c["layers"][1]["mixer"]["right"].update(tau=0.0),
+    ],
+)
+def test_config_refuses_what_does_not_fit(change):
+    cfg = json.loads(json.dumps(CONFIGS["A"]))
+    change(cfg)
+    with pytest.raises(ConfigError):
+        config_from_dict(cfg)
+
+
+def test_model_is_built_from_the_framework_parts(tmp_path):
+    from mini_llm_runtime_amd.cache import CompositeSpec, PagedKVSpec, SlotStateSpec
+
+    model = build_model(config_from_dict(CONFIGS["A"]))
+    kinds = [(type(l).__name__, type(l.mixer).__name__, type(l.feed_forward).__name__) for l in model.layers]
+    assert kinds == [("ParallelBlock", "SideBySide", "SwiGLU"), ("ParallelBlock", "SideBySide", "NoneType")]
+    assert [type(m).__name__ for m in model.layers[0].mixer.members.values()] == ["PooledWindowAttention", "GatedLinearAttention"]
+    assert model.replayable
+    specs = model.site_cache_specs()
+    assert len(specs) == 3  # the looped layer's two runs keep caches of their own
+    assert specs[0] == specs[1] and specs[0] != specs[2]
+    first = specs[0]
+    assert isinstance(first, CompositeSpec)
+    assert first.members["filter"] == SlotStateSpec((3, 64), "float32")
+    mixer = first.members["mixer"]
+    assert mixer.members["right"] == SlotStateSpec((2, 16, 32), "float32")
+    left = mixer.members["left"]
+    assert left.members["tokens"] == PagedKVSpec(2, 32, 10)  # keys of 16 and values of 24 in pages of 32 dims
+    assert left.members["pooled"] == PagedKVSpec(2, 32, tokens_per_entry=4)
+    # loaded beside a checkpoint, the decay's inner size is the stored tensor's
+    folder, _, _ = make_dir(tmp_path, "A")
+    from mini_llm_runtime_amd import load_model
+
+    _, loaded = load_model(folder, dtype=torch.float32, device="cpu")
+    assert loaded.layers[0].mixer.members["right"].decay_rank == 5 and loaded.layers[1].mixer.members["right"].decay_rank == 16
+
+
+# ---- mechanisms alone, on the GPU ----------------------------------------------------------------------
+
+def _ctx(lens, starts):
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    entry = [i for i, n in enumerate(lens) for _ in range(n)]
+    positions = [s + j for s, n in zip(starts, lens) for j in range(n)]
+    as_int = lambda x: torch.tensor(x, dtype=torch.int32).cuda()  # noqa: E731
+    return SimpleNamespace(
+        num_entries=len(lens), cu_q=as_int(cu), q_starts=as_int(starts), token_entry=as_int(entry), positions=as_int(positions),
+    ), cu
+
+
+@pytest.mark.parametrize("dtype", GPU_CASES)
+@pytest.mark.parametrize("width,taps,add", [(64, 4, True), (70, 2, True), (300, 3, False), (16, 1, True), (520, 5, True)])
+def test_short_convolution_with_carried_inputs(dtype, width, taps, add):
+    """Entries of 1, 2, 5 and 70 tokens: two start their request (whatever the row holds), two go on from carried
+    inputs, one of them from a request shorter than the taps; rows of other slots stay."""
+    ops = _ops("hip", dtype)
+    g = torch.Generator().manual_seed(width + taps)
+    lens, starts = [2, 1, 70, 5], [0, 2, 9, 0]
+    ctx, cu = _ctx(lens, starts)
+    h = torch.randn(sum(lens), width, generator=g).to(dtype)
+    w = (torch.randn(width, taps, generator=g) * 0.5).to(dtype)
+    history = [torch.randn(s, width, generator=g).to(dtype).float() for s in starts]
+    carried = taps - 1
+    bank = torch.randn(9, max(carried, 1), width, generator=g)
+    read, write = [0, 3, 4, 6], [1, 2, 5, 7]
+    for r, hist in enumerate(history):
+        if hist.shape[0] and carried:
+            bank[read[r]] = torch.cat([torch.zeros(carried, width), hist])[-carried:]
+    state = bank[:, :carried].contiguous().cuda() if carried else None
+    as_int = lambda x: torch.tensor(x, dtype=torch.int32).cuda()  # noqa: E731
+    out = ops.short_conv(h.cuda(), w.cuda(), state, as_int(read), as_int(write), ctx, add_input=add)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    for r in range(4):
+        rows = h[cu[r] : cu[r + 1]].double()
+        seq = torch.cat([history[r].double(), rows])
+        want = plain.causal_conv(seq, w.double())[-lens[r] :] + (rows if add else 0.0)
+        torch.testing.assert_close(out[cu[r] : cu[r + 1]].double().cpu(), want, **tol)
+        if carried:
+            left = torch.cat([torch.zeros(carried, width, dtype=torch.float64), seq])[-carried:]
+            torch.testing.assert_close(state[write[r]].double().cpu(), left, rtol=0, atol=0)
+    if carried:
+        for row in set(range(9)) - set(write):
+            assert torch.equal(state[row].cpu(), bank[row, :carried]), f"row {row} was written"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(2, 16, 32, 5, 8.0), (3, 20, 12, 16, 1.0), (4, 64, 48, 8, 16.0), (1, 128, 16, 3, 2.0), (2, 200, 20, 1, 64.0)])
+def test_decayed_recurrence_and_its_state_rows(heads, dim, vdim, rank, tau):
+    """Three entries of unequal length (one token, a few, two chunks of 64 and a bit), two of which go on from a
+    carried state; rows of other slots stay.  Then the heads' norm with its shared weight and the gate."""
+    ops = _ops("hip", torch.float32)
+    g = torch.Generator().manual_seed(heads * dim + vdim)
+    lens, starts = [5, 1, 150], [0, 40, 7]
+    ctx, cu = _ctx(lens, starts)
+    tokens = sum(lens)
+    qk, out_w = heads * dim, heads * vdim
+    width = 2 * qk + 2 * out_w + rank
+    p = torch.randn(tokens, width, generator=g)
+    w2 = torch.randn(qk, rank, generator=g) * 2.0
+    bias = torch.randn(qk, generator=g) * 2.0 + 2.0
+    bank = torch.randn(10, heads, dim, vdim, generator=g)  # stale values everywhere
+    read, write = [0, 3, 4], [1, 2, 5]
+    state = bank.clone().cuda()
+    as_int = lambda x: torch.tensor(x, dtype=torch.int32).cuda()  # noqa: E731
+    out = ops.gla_scan(
+        p.cuda(), state, as_int(read), as_int(write), ctx, heads=heads, head_dim=dim, value_dim=vdim,
+        decay_weight=w2.cuda(), decay_bias=bias.cuda(), low_offset=2 * qk + 2 * out_w, tau=tau, q_scale=dim**-0.5,
+    )
+    for r in range(3):
+        rows = p[cu[r] : cu[r + 1]].double()
+        q = (rows[:, :qk] * dim**-0.5).view(-1, heads, dim)
+        k = rows[:, qk : 2 * qk].view(-1, heads, dim)
+        v = rows[:, 2 * qk : 2 * qk + out_w].view(-1, heads, vdim)
+        alpha = torch.sigmoid(rows[:, 2 * qk + 2 * out_w :] @ w2.double().T + bias.double()).pow(1.0 / tau).view(-1, heads, dim)
+        s = bank[read[r]].double() if starts[r] > 0 else torch.zeros(heads, dim, vdim, dtype=torch.float64)
+        for t in range(lens[r]):
+            s = alpha[t][:, :, None] * s + k[t][:, :, None] * v[t][:, None, :]
+            want = torch.einsum("hdv,hd->hv", s, q[t]).reshape(-1)
+            torch.testing.assert_close(out[cu[r] + t].double().cpu(), want, rtol=2e-4, atol=2e-4)
+        torch.testing.assert_close(state[write[r]].double().cpu(), s, rtol=2e-4, atol=2e-4)
+    for row in set(range(10)) - set(write):
+        assert torch.equal(state[row].cpu(), bank[row]), f"row {row} was written"
+    norm_w = 1.0 + 0.3 * torch.randn(vdim, generator=g)
+    gated = ops.retention_gate(
+        out, p.cuda(), heads=heads, value_dim=vdim, gate_offset=2 * qk + out_w, eps=1e-5, norm_weight=norm_w.cuda(), scale=0.7,
+    )
+    z = p[:, 2 * qk + out_w : 2 * qk + 2 * out_w].double()
+    want = plain.rms_norm(out.double().cpu().view(tokens, heads, vdim), norm_w.double(), 1e-5).reshape(tokens, -1) * (z * torch.sigmoid(z)) * 0.7
+    torch.testing.assert_close(gated.double().cpu(), want, rtol=1e-4, atol=1e-4)
+
+
+# ---- one key that holds the weight, at every edge ---------------------------------------------------------
+
+def _needle_model(window: int, pool: int, dim: int, vdim: int, sink: float, scale: float, taps: int = 2) -> tuple[dict, dict]:
+    """One layer whose recurrent half counts nothing, with one attention head made so that a query's weight
+    sits on ONE key wherever it lies: token 1 marks a key, token 2 asks, every other token is filler whose key
+    is at right angles to the question.  The dims that carry this do not turn, so the distance does not matter.
+    The marked key's value goes into the logits, so they say whether that key was seen."""
+    width = 16
+    left = _left(1, 1, dim, vdim, window, pool, dim // 2, 2.0, scale)
+    cfg = _model(8, width, 1e-6, 1.0, taps, [_layer(left, _right(1, 8, 8, 2.0), None, 1.0, 0.0)])
+    g = torch.Generator().manual_seed(window + pool)
+    w = {k: v.float() for k, v in make_weights(cfg, 5).items()}
+    w["embed"] = torch.zeros(8, width)
+    w["embed"][:, :8] = torch.eye(8) * 4.0
+    w["l0.norm1"] = torch.ones(width)
+    w["l0.canon1"] = torch.zeros(width, taps)  # a token's key is its own
+    q = torch.zeros(dim, width)
+    q[dim - 1, 2] = 8.0  # the query of token 2 ...
+    k = torch.randn(dim, width, generator=g) * 0.02
+    k[dim - 1, 1] = 8.0  # ... meets the key of token 1
+    k[dim - 2, 2:8] = 8.0  # everybody else's key points elsewhere
+    p = "l0.mix.left."
+    w[p + "q"], w[p + "k"] = q, k
+    w[p + "q.b"], w[p + "k.b"] = torch.zeros(dim), torch.zeros(dim)
+    w[p + "q.norm"], w[p + "k.norm"] = torch.ones(dim), torch.ones(dim)
+    w[p + "temp"] = torch.ones(1)
+    w[p + "v"] = torch.randn(vdim, width, generator=g) * 0.5
+    w[p + "g"] = torch.zeros(1, width)
+    w[p + "sink"] = torch.tensor([sink])
+    w[p + "o"] = torch.randn(width, vdim, generator=g) * 0.5
+    return cfg, {name: t.to(torch.bfloat16) for name, t in w.items()}
+
+
+# (window, pooled block, length, where the marked key lies counted back from the query, what it is)
+_EDGES = [
+    (10, 4, 40, 9, "the oldest token of the window"),
+    (10, 4, 40, 10, "just out of the window, its block not complete"),
+    (10, 4, 41, 10, "just out of the window, the last of a block that is seen from now on"),
+    (10, 4, 41, 13, "the first token of the block that is seen from now on"),
+    (10, 4, 40, 12, "the first token of a block whose last is still in the window"),
+    (10, 4, 40, 39, "the very first token, in the first pooled block"),
+    (7, 16, 66, 22, "a block as long as a page, seen from now on"),
+    (7, 16, 65, 21, "the same block one step earlier: not seen, though most of it left the window"),
+    (20, 3, 700, 640, "hundreds of tokens back"),
+    (300, 8, 420, 299, "the oldest token of a window that spans many pages"),
+    (300, 8, 420, 300, "just out of it, in a block that is not complete"),
+    (5, 8, 30, 4, "a window shorter than the block: its oldest token"),
+    (5, 8, 28, 12, "a window shorter than the block: the newest block's first token"),
+]
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("window,pool,length,back,what", _EDGES)
+def test_one_key_at_every_edge(tmp_path, backend, dtype, window, pool, length, back, what):
+    """Queries at the end of a prompt, of a portion, and decoded alone (after other tokens decoded alone, so the
+    window has passed over decoded tokens)."""
+    if backend == "double" and length > 150:
+        pytest.skip("the CPU stand-in is slow at this length")
+    cfg, weights = _needle_model(window, pool, 16, 24, sink=-2.0, scale=4.0)
+    folder = write_model(tmp_path, "needle", cfg, weights)
+    ask = length - 1
+    marked = ask - back
+    # by the rule itself: in the window, or in a block that lies wholly before it
+    seen = back < window or (marked // pool) * pool + pool - 1 <= ask - window
+    cases = {}
+    for name, token in (("marked", 1), ("unmarked", 3)):
+        toks = [3 + (i % 5) for i in range(length)]
+        toks[marked] = token
+        toks[ask] = 2
+        cases[name] = toks
+    refs = {name: plain.forward(cfg, weights, toks)[-1] for name, toks in cases.items()}
+    differ = float((refs["marked"] - refs["unmarked"]).abs().max()) / float(refs["marked"].abs().max())
+    assert (differ > 0.03) == seen and (seen or differ < 1e-9), f"{what}: the plain logits differ by {differ:.3f}"
+    ops = _ops(backend, dtype)
+    tail = min(length - 1, window + pool + 3)
+    _, _, cache, runner = make_runner(folder, ops, block_size=16, num_blocks=2 * (length // 16 + 2), max_requests=2)
+    cache.poison()
+    for family in (schedules.whole, lambda r: schedules.bulk_then_tail(r, tail=tail), schedules.portions):
+        got = schedules.run_schedule(runner, cache, family(cases))
+        for name in cases:
+            row = got[(name, ask)].double()
+            assert float((row - refs[name]).abs().max()) < (1e-4 if dtype == torch.float32 else 0.08) * float(refs[name].abs().max()), what
+        gap = float((got[("marked", ask)] - got[("unmarked", ask)]).abs().max()) / float(got[("marked", ask)].abs().max())
+        assert (gap > 0.03) if seen else (gap < 1e-6), f"{what}: {gap:.3f}"
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+def test_sinks_that_take_most_of_one_head(tmp_path, backend, dtype):
+    """Two heads, one of which loses nearly all its weight to its sink.  Left out, swapped between the heads,
+    scaled like a score, or counted once per partition of the keys, the logits differ."""
+    length = 330
+    cfg = _model(96, 32, 1e-6, 2.0, 2, [_layer(_left(2, 1, 16, 16, 290, 8, 8, None, 0.2), _right(1, 8, 8, 2.0), None, 1.0, 0.0)])
+    toks = random_tokens(length, 96, 21)
+    results = {}
+    for sinks in ((25.0, -25.0), (-25.0, 25.0)):
+        weights = make_weights(cfg, 13)
+        weights["l0.mix.left.sink"] = torch.tensor(sinks).to(torch.bfloat16)
+        weights["l0.mix.left.temp"] = torch.tensor([0.5, 3.0]).to(torch.bfloat16)  # a sink times this would show
+        ref = results[sinks] = plain.forward(cfg, weights, toks)[-1]
+        if backend == "double" and sinks[0] < 0:
+            continue
+        folder = write_model(tmp_path, f"sink{int(sinks[0])}", cfg, weights)
+        ops = _ops(backend, dtype)
+        _, _, cache, runner = make_runner(folder, ops, block_size=16, num_blocks=length // 16 + 2, max_requests=1)
+        for family in (schedules.whole, lambda r: schedules.bulk_then_tail(r, tail=3)):
+            got = schedules.run_schedule(runner, cache, family({"a": toks}))
+            row = got[("a", length - 1)].double()
+            assert float((row - ref).abs().max()) < (1e-4 if dtype == torch.float32 else 0.08) * float(ref.abs().max())
+    a, b = results.values()
+    assert float((a - b).abs().max()) > 0.2 * float(a.abs().max())
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+def test_a_state_that_remembers_the_first_token(tmp_path, backend, dtype):
+    """A recurrent head whose decay is all but 1 in every channel: the first token's key and value stay in the
+    state, so a state lost between two steps, or a slot cleared too late, shows at every later position."""
+    cfg = CONFIGS["R"]
+    weights = make_weights(cfg, 11, RANKS["R"])
+    weights["l0.mix.right.a2.b"] = torch.full((32,), 9.0).to(torch.bfloat16)
+    weights["l0.mix.right.a2"] = (weights["l0.mix.right.a2"].float() * 0.1).to(torch.bfloat16)
+    folder = write_model(tmp_path, "keeper", cfg, weights)
+    a = random_tokens(90, 128, 1)
+    b = [(a[0] + 1) % 128] + a[1:]  # differs in the first token only
+    ref_a, ref_b = plain.forward(cfg, weights, a), plain.forward(cfg, weights, b)
+    # the oracle remembers: clearly at the twentieth token (where a portion or the bulk's end may fall), still at the last
+    assert float((ref_a[20] - ref_b[20]).abs().max()) > 0.1 * float(ref_a[20].abs().max())
+    assert float((ref_a[-1] - ref_b[-1]).abs().max()) > 0.01 * float(ref_a[-1].abs().max())
+    ops = _ops(backend, dtype)
+    _, _, cache, runner = make_runner(folder, ops, block_size=4, num_blocks=48, max_requests=1)
+    for family in (schedules.whole, lambda r: schedules.bulk_then_tail(r, tail=40), schedules.portions):
+        for name, toks in (("a", a), ("b", b), ("a", a)):  # one slot, used again and again
+            got = schedules.run_schedule(runner, cache, family({name: toks}))
+            _compare(got, {name: toks}, weights, cfg, dtype)
+
+
+# ---- whole models under every schedule -------------------------------------------------------------------
+
+FAMILIES = {
+    "whole": schedules.whole,
+    "bulk_then_tail": lambda r: schedules.bulk_then_tail(r, tail=48),
+    "portions": schedules.portions,
+    "mixed": schedules.mixed,
+    "mixed_two_slots": lambda r: schedules.mixed(r, max_live=2, seed=5, decode_tail=20),
+}
+
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("family", list(FAMILIES))
+@pytest.mark.parametrize("which", list(CONFIGS))
+def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
+    if backend == "double" and (which == "D" or (which == "C" and family != "mixed")):
+        pytest.skip("the CPU stand-in is slow at this size")
+    folder, cfg, weights = make_dir(tmp_path, which)
+    requests = _requests(which)
+    steps = FAMILIES[family](requests)
+    bs = BLOCK[which]
+    _, model, cache, runner = make_runner(
+        folder, _ops(backend, dtype), block_size=bs, num_blocks=max(1, schedules.pages_needed(steps, bs)),
+        max_requests=schedules.most_live(steps),
+    )
+    cache.poison()
+    for bank in cache.state_banks.values():  # stale states in every slot: a request must start from zeros
+        bank.tensor.fill_(float("nan"))
+    got = schedules.run_schedule(runner, cache, steps)
+    _compare(got, requests, weights, cfg, dtype)
+    cache.check_invariants()
+    assert all(g.allocator.free_count == g.num_blocks for g in cache.groups), "pages were not given back"
+
+
+def test_layer_outputs_match_plain(tmp_path):
+    folder, cfg, weights = make_dir(tmp_path, "A")
+    toks = random_tokens(31, cfg["vocab"], 8)
+    _, _, cache, runner = make_runner(folder, _ops("double", torch.float32), block_size=16, num_blocks=4, max_requests=1)
+    cache.create_request("a")
+    from helpers import StepEntry
+
+    out = runner.step([StepEntry.of("a", toks, [0, 17, 30])], capture_sites=True)
+    _, layers = plain.forward(cfg, weights, toks, return_layers=True)
+    assert out.site_outputs.shape == (3, 3, cfg["width"])  # the looped layer counts each time
+    for i, x in enumerate(layers):
+        torch.testing.assert_close(out.site_outputs[i].double(), x[[0, 17, 30]], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", GPU_CASES)
+def test_replayed_steps_equal_plain_steps(tmp_path, dtype):
+    """Steps of a model with state slots, carried inputs and two kinds of pages are recorded and replayed; the
+    replays give what the unrecorded steps give, bit for bit."""
+    folder, cfg, _ = make_dir(tmp_path, "C")
+    requests = {"a": random_tokens(90, cfg["vocab"], 1), "b": random_tokens(75, cfg["vocab"], 2)}
+    steps = schedules.bulk_then_tail(requests, tail=40)
+    results = []
+    for use_graphs in (False, True):
+        _, _, cache, runner = make_runner(folder, _ops("hip", dtype), block_size=16, num_blocks=16, max_requests=2)
+        runner.use_graphs = use_graphs
+        results.append(schedules.run_schedule(runner, cache, steps))
+    plain_steps, replayed = results
+    assert plain_steps.keys() == replayed.keys()
+    for key in plain_steps:
+        assert torch.equal(plain_steps[key], replayed[key]), key
+
+
+# ---- generation through the engine ------------------------------------------------------------------------
+
+@pytest.mark.parametrize("backend,dtype", CASES)
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_generation_through_the_engine(tmp_path, which, backend, dtype):
+    folder, cfg, weights = make_dir(tmp_path, which)
+    ops = _ops(backend, dtype)
+    engine = ContinuousBatchEngine.from_model_dir(
+        folder, dtype=ops.dtype, ops=ops, block_size=BLOCK[which], num_blocks=40, max_running_requests=3,
+        max_batch_tokens=24,
+    )
+    prompts = [random_tokens(n, cfg["vocab"], 9 + n) for n in (5, 30, 1, 17)]
+    outs = engine.generate(prompts, max_new_tokens=40)  # long enough for the window to pass over decoded tokens
+    for prompt, tokens in zip(prompts, outs):
+        assert len(tokens) == 40
+        seq = list(prompt)
+        for i, tok in enumerate(tokens):
+            logits = plain.forward(cfg, weights, seq)[-1]
+            best = int(torch.argmax(logits))
+            if tok != best:
+                # only rounding may choose between two nearly equal logits, and only in bfloat16
+                assert dtype == torch.bfloat16, f"token {i}: {tok} != {best}"
+                assert float(logits[best] - logits[tok]) < 6e-2 * float(logits.abs().max())
+                break
+            seq.append(tok)
+
+
+# ---- the command line and the replay program --------------------------------------------------------------
+
+def test_preset_and_random_model_writer(tmp_path):
+    from helpers import read_weights
+    from mini_llm_runtime_amd import cli
+    from mini_llm_runtime_amd.config.presets import load_preset, preset_names
+
+    assert "vobisun-tiny" in preset_names()
+    assert cli.main(["random-model", "--config", "vobisun-tiny", "--seed", "2", "--out", str(tmp_path / "m")]) == 0
+    cfg, w = read_weights(tmp_path / "m")
+    preset = load_preset("vobisun-tiny")
+    first = preset["layers"][0]["mixer"]
+    assert cfg["architecture"] == "Vobisun" and w["embed"].shape == (preset["vocab"], preset["width"])
+    assert w["l0.mix.left.q"].shape == (first["left"]["heads"] * first["left"]["dim"], preset["width"])
+    assert w["l0.mix.left.sink"].shape == (first["left"]["heads"],) and w["l0.canon1"].shape == (preset["width"], preset["canon"]["taps"])
+    assert w["l0.mix.right.a2"].shape[0] == first["right"]["heads"] * first["right"]["dim"]
+    assert ("l1.mlp.gate" in w) == (preset["layers"][1]["mlp"] is not None)
+    plain.forward(cfg, w, [1, 2, 3])  # the plain implementation reads the same folder
+
+
+@pytest.mark.gpu
+def test_generate_command_and_trace_replay(tmp_path, gpu_device):
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    folder, cfg, weights = make_dir(tmp_path, "A")
+    prompt = random_tokens(21, cfg["vocab"], 4)
+    proc = subprocess.run(
+        [sys.executable, "-m", "mini_llm_runtime_amd.cli", "generate", "--model", str(folder), "--dtype", "float32",
+         "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5"],
+        cwd=ROOT, capture_output=True, text=True, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    out = json.loads(proc.stdout.strip().splitlines()[-1])
+    seq = list(prompt)
+    for tok in out["generated_token_ids"]:
+        assert tok == int(torch.argmax(plain.forward(cfg, weights, seq)[-1]))
+        seq.append(tok)
+    # the replay program: requests in portions beside each other, slots and pages used again
+    toks = {"a": random_tokens(40, cfg["vocab"], 5), "b": random_tokens(27, cfg["vocab"], 6), "c": random_tokens(33, cfg["vocab"], 7)}
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks["a"][:25], "want": [0, 24]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks["a"][25:27], "want": [1]}, {"id": "b", "tokens": toks["b"], "want": [26]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks["a"][27:], "want": [12]}, {"id": "c", "tokens": toks["c"][:32], "want": []}], "end": ["a"]},
+        {"step": 3, "entries": [{"id": "c", "tokens": toks["c"][32:], "want": [0]}], "end": ["c"]},
+    ]
+    for dtype in ("bfloat16", "float32"):
+        proc = subprocess.run(
+            [str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype, "--out", str(tmp_path / dtype),
+             "--max-tokens", "128", "--max-live", "2"],
+            input="".join(json.dumps(s) + "\n" for s in steps), cwd=ROOT, capture_output=True, text=True, timeout=300,
+        )
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+        wanted = {0: [("a", 0), ("a", 24)], 1: [("a", 26), ("b", 26)], 2: [("a", 39)], 3: [("c", 32)]}
+        for step, rows in wanted.items():
+            got = torch.from_numpy(np.fromfile(tmp_path / dtype / f"{step}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"]))
+            for row, (rid, pos) in zip(got, rows):
+                ref = plain.forward(cfg, weights, toks[rid][: pos + 1])[-1]
+                rel = float((row.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt())
+                assert rel < (6e-2 if dtype == "bfloat16" else 1e-4), (step, rid, pos, rel)
