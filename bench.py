@@ -44,6 +44,9 @@ feed-forward) beside the Qwen2 decoder at equal sizes (`DESIGN_POINTS`): decode 
 `hybrid-*` (`BUBITAR_POINTS`; not among the default points) run the Bubitar decoder (retention layers and
 latent-attention layers in turn, sandwich norms, clamped gated feed-forward, a token input per layer) beside
 the Qwen2 decoder of the same width, heads, head size, feed-forward width, layers and vocabulary.
+The points named `side-*` (`VOBISUN_POINTS`; not among the default points either) run the Vobisun decoder
+(parallel layers whose mixer is windowed attention with pooled blocks beside linear attention with a decay
+per key channel, a short convolution before the mixer, a looped span of layers) beside that same Qwen2 twin.
 `reference`: the reference's own published measurements, run here at their parameters with the
 0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
 laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and
@@ -103,7 +106,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference", "designs"))
-    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2", "bubitar"), help="run one of the two designs of the `designs` workload (for profiles)")
+    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2", "bubitar", "vobisun"), help="run one of the two designs of the `designs` workload (for profiles)")
     p.add_argument("--design-points", default="", help="names of the `designs` workload's points to run, comma separated (default: all)")
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
@@ -785,6 +788,21 @@ class Bench:
                 + 2 * config.vocab_size * config.hidden_size
             )
         width, flops = config.width, 2 * config.vocab * config.width
+        if hasattr(config, "canon_taps"):
+            # per layer run: the attention half's input and output products and its (query, visible key) pairs
+            # (the window's tokens and the pooled blocks before it), the recurrent half's products, its decay's
+            # small product and the state update and read (2 x dim x vdim a head and token), the feed-forward
+            for i in config.layer_runs():
+                layer = config.layers[i]
+                a, b = layer.left, layer.right
+                per_token = width * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + a.heads) + a.heads * a.vdim * width
+                per_token += width * (2 * b.heads * b.dim + 2 * b.heads * b.vdim + b.rank) + b.rank * b.heads * b.dim
+                per_token += 2 * b.heads * b.dim * b.vdim + b.heads * b.vdim * width
+                if layer.ff is not None:
+                    per_token += 3 * width * layer.ff
+                pairs = sum(min(t + 1, a.window) + max(0, t - a.window + 1) // a.pool for t in range(tokens))
+                flops += 2 * tokens * per_token + 2 * a.heads * (a.dim + a.vdim) * pairs
+            return flops
         if hasattr(config, "token_side_dim"):
             # retention: four input products, the state update and read (2 x dim x vdim a head and token, as the
             # recurrence counts them), the output product; latent attention as the kernels run it: input
@@ -912,9 +930,52 @@ def bubitar_configs(name: str) -> dict:
     return {"bubitar": bubitar, "qwen2": qwen2}
 
 
+# The Vobisun decoder beside the Qwen2 decoder: the same width, query and key/value heads, head size, feed-forward
+# width, layer runs and vocabulary.  The attention half keeps a window of 1,024 tokens and one pooled entry for
+# every 64 older ones (half of a head's dims turn); the recurrent half has half as many heads, keys of the head size
+# and values of twice that, so both halves hand the same number of activations to the one output product.  Two of
+# the listed layers run twice.
+VOBISUN_POINTS = {
+    # name: (width, heads, kv heads, head size, feed-forward width, layer runs)
+    "side-0.5b": (896, 14, 2, 64, 4864, 12),
+    "side-7b": (3584, 28, 4, 128, 18944, 4),
+}
+
+
+def vobisun_configs(name: str) -> dict:
+    width, heads, kv_heads, dim, inter, runs = VOBISUN_POINTS[name]
+    layer = {
+        "type": "parallel",
+        "mixer": {
+            "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim**-0.5,
+                     "mask": {"size": 1024, "pool": 64},
+                     "rot": {"base": 1000000.0, "dims": dim // 2, "scaling": {"factor": 4.0}}},
+            "left_scale": 1.0,
+            "right": {"heads": heads // 2, "dim": dim, "vdim": 2 * dim, "tau": 16.0},
+            "right_scale": 1.0,
+        },
+        "mlp": {"kind": "dense", "ff": inter},
+    }
+    vobisun = {
+        "architecture": "Vobisun", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5},
+        "embedding": {"scale": 1.0}, "canon": {"taps": 4},
+        "loop": {"start": min(1, runs - 4), "stop": min(1, runs - 4) + 2, "times": 2},
+        "layers": [json.loads(json.dumps(layer)) for _ in range(runs - 2)],
+    }
+    qwen2 = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": DESIGN_VOCAB, "hidden_size": width,
+        "intermediate_size": inter, "num_hidden_layers": runs, "num_attention_heads": heads,
+        "num_key_value_heads": kv_heads, "head_dim": dim, "max_position_embeddings": 32768, "rms_norm_eps": 1e-5,
+        "rope_theta": 1000000.0, "hidden_act": "silu", "tie_word_embeddings": True,
+    }
+    return {"vobisun": vobisun, "qwen2": qwen2}
+
+
 def design_configs(name: str) -> dict:
     if name in BUBITAR_POINTS:
         return bubitar_configs(name)
+    if name in VOBISUN_POINTS:
+        return vobisun_configs(name)
     width, heads, kv_heads, dim, inter, layers, mlp = DESIGN_POINTS[name]
     fedolorn = {
         "architecture": "Fedolorn", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5},
@@ -954,7 +1015,7 @@ def design_comparison(args) -> dict:
                 "prefill_ms": prefill["ms"],
                 "prefill_frac_of_peak": prefill["frac"],
                 "weight_bytes": int(weight_bytes),
-                "layers": len(bench.model.layers),
+                "layers": len(bench.model.spec.order) if bench.model.spec.order else len(bench.model.layers),
             }
             bench.close()
             print(f"# {name} {design}: {point[design]}", file=sys.stderr, flush=True)
