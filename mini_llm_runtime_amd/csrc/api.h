@@ -236,6 +236,14 @@ int mlr_pool_kv_write(const void* key_pages, const void* value_pages, const int*
                       void* pooled_keys, void* pooled_values, int pooled_pages, int dtype, int tokens, int kv_heads,
                       int head_dim, int block_size, int pool, hipStream_t stream);
 
+// The pooled entries' share of a softmax that the matrix-core attention kernels finish (their `extra`): for every
+// token and head, over the entries j < (position - window + 1) / pool of the entry's pooled pages, share[t, h] =
+// [numerator (head_dim floats), maximum of score * scale * log2(e), denominator]; bfloat16 queries and pages.
+int mlr_pooled_share(const void* q, int64_t q_stride, const void* pooled_keys, const void* pooled_values,
+                     const int* pooled_table, int table_width, int pooled_pages, const int* token_entry,
+                     const int* positions, float* share, int tokens, int heads, int kv_heads, int head_dim,
+                     int block_size, float scale, int window, int pool, hipStream_t stream);
+
 // out[t * out_row + head * out_dim + j] = attended[t, head * head_dim + j] * gate[t, head] * scale, j < out_dim.
 int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t out_row, int dtype, int tokens, int heads,
                     int head_dim, int out_dim, float scale, hipStream_t stream);

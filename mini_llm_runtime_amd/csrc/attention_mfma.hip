@@ -176,7 +176,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ partial, int heads, int kv_heads, int head_tiles, int block_size, int num_pages,
-    float scale, int window, int chunk, int part, int splits, const float* __restrict__ sinks) {
+    float scale, int window, int chunk, int part, int splits, const float* __restrict__ sinks, int keep_partial) {
   __shared__ float sm_acc[kDecodeWaves][16][D];
   __shared__ float sm_m[kDecodeWaves][16];
   __shared__ float sm_l[kDecodeWaves][16];
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       den += wgt * sm_l[w][c];
     }
     const int h = kvh * group + htile * 16 + c;
-    if (splits == 1) {
+    if (splits == 1 && !keep_partial) {
       num *= join_sink(sinks, h, mstar, den);  // with partitions the merge does this, once
       const float v = poisoned ? __builtin_nanf("") : num / den;
       out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(v);
@@ -350,7 +350,8 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
                                                                   const int* __restrict__ context_lens,
                                                                   bf16* __restrict__ out, int heads, int window,
                                                                   int chunk, int part, int all_splits,
-                                                                  const float* __restrict__ sinks) {
+                                                                  const float* __restrict__ sinks,
+                                                                  const float* __restrict__ extra) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -408,6 +409,22 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
     s0 += kMergeBatch;
     if (s0 >= splits) break;
     load_batch(s0);
+  }
+  if (extra != nullptr) {  // one more share of the same softmax, made elsewhere: [token, head, head size + 2]
+    const float* e = extra + (static_cast<int64_t>(t) * heads + h) * kPartialStride;
+    const float m_e = e[D];
+    if (m_e != -INFINITY) {
+      const float m_new = fmaxf(mstar, m_e);
+      const float mine = (mstar == -INFINITY) ? 0.f : fast_exp2(mstar - m_new);
+      const float theirs = fast_exp2(m_e - m_new);
+#pragma unroll
+      for (int j = 0; j < kPerLane; ++j) {
+        const int d = lane + j * kWave;
+        num[j] = num[j] * mine + (d < D ? e[d] : 0.f) * theirs;
+      }
+      den = den * mine + e[D + 1] * theirs;
+      mstar = m_new;
+    }
   }
   const float keep = join_sink(sinks, h, mstar, den);
 #pragma unroll
@@ -471,7 +488,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
-    int window, int chunk, float* __restrict__ partial, const float* __restrict__ sinks) {
+    int window, int chunk, float* __restrict__ partial, const float* __restrict__ sinks, int keep_partial) {
   // gridDim.y > 1: the keys of every tile are cut into that many runs, one workgroup each, which
   // leave their unnormalised results in `partial` for attn_prefill_merge (few tiles behind a long
   // context would otherwise be as many long chains on a few compute units).
@@ -823,7 +840,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     float l = l_run[b];
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
-    if (splits > 1) {
+    if (splits > 1 || keep_partial) {
       // this run's share, unnormalised: [tile, head, run, query of the tile, head size + 2]
       float* dst = partial + (((static_cast<int64_t>(tile) * heads + head) * splits + blockIdx.y) * kWgQ +
                               (wave * kWaveQ + b * 16 + col)) * kPartialStride;
@@ -865,7 +882,8 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
                                                                  const int* __restrict__ tiles,
                                                                  const int* __restrict__ cu_q,
                                                                  bf16* __restrict__ out, int heads, int splits,
-                                                                 int tile_q, const float* __restrict__ sinks) {
+                                                                 int tile_q, const float* __restrict__ sinks,
+                                                                 const float* __restrict__ extra) {
   const int tile = blockIdx.x / heads;
   const int head = blockIdx.x - tile * heads;
   const int entry = tiles[2 * tile];
@@ -889,6 +907,19 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
       num1 += w * row[d + 1];
       den += w * row[D + 1];
     }
+    if (extra != nullptr) {  // one more share of the same softmax, made elsewhere: [token, head, head size + 2]
+      const float* e = extra + (static_cast<int64_t>(t_first + q0 + qq) * heads + head) * kPartialStride;
+      const float m_e = e[D];
+      if (m_e != -INFINITY) {
+        const float m_new = fmaxf(mstar, m_e);
+        const float mine = (mstar == -INFINITY) ? 0.f : fast_exp2(mstar - m_new);
+        const float theirs = fast_exp2(m_e - m_new);
+        num0 = num0 * mine + e[d] * theirs;
+        num1 = num1 * mine + e[d + 1] * theirs;
+        den = den * mine + e[D + 1] * theirs;
+        mstar = m_new;
+      }
+    }
     const float keep = join_sink(sinks, head, mstar, den);
     bf16* orow = out + (static_cast<int64_t>(t_first + q0 + qq) * heads + head) * D;
     orow[d] = f32_to_bf16(num0 * keep / den);
@@ -907,9 +938,10 @@ int mlr_attention_head_dim() { return D; }
 // Key positions per LDS tile of the prefill kernel; block_size must divide it.
 int mlr_attention_key_tile() { return kTileK; }
 
-// Floats of scratch the decode kernel needs for `splits` partitions.
+// Floats of scratch the decode kernel needs for `splits` partitions (one partition writes none unless a
+// share made elsewhere joins its softmax, see `extra`).
 int64_t mlr_attention_decode_scratch(int entries, int heads, int splits) {
-  return splits <= 1 ? 0 : static_cast<int64_t>(entries) * heads * splits * kPartialStride;
+  return splits < 1 ? 0 : static_cast<int64_t>(entries) * heads * splits * kPartialStride;
 }
 
 // Attention of every single-token entry (entries with more tokens are skipped).
@@ -918,24 +950,29 @@ int64_t mlr_attention_decode_scratch(int entries, int heads, int splits) {
 // mlr_attention_decode_scratch floats, laid out [entry, head, split, head size + 2]
 // (numerator, maximum in base 2, denominator).  `merge` 0 leaves the partitions unmerged in
 // `partial` for a consumer that merges them itself (or for mlr_attention_decode_merge).
+// `extra` (or null): float32 [tokens, heads, head size + 2], for every token and head one more share of the same
+// softmax in the partitions' form (numerator, maximum of score * scale * log2(e), denominator; a maximum of
+// -infinity: nothing), made by another kernel over other keys; the merge takes it in before the sink.
 int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* context_lens,
                          void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
                          int num_pages, float scale, int window, int chunk, int part, int splits, int merge,
-                         const float* sinks, hipStream_t stream) {
+                         const float* sinks, const float* extra, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
   MLR_REQUIRE(block_size > 0 && block_size % 4 == 0, "block_size must be a multiple of 4");
   MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
   MLR_REQUIRE(part > 0 && part % 64 == 0, "part must be a positive multiple of 64");
   MLR_REQUIRE(splits >= 1 && splits <= 65535, "splits out of range");
-  MLR_REQUIRE(splits == 1 || partial != nullptr, "several partitions need scratch memory");
+  MLR_REQUIRE((splits == 1 && extra == nullptr) || partial != nullptr, "several partitions, or a share made elsewhere, need scratch memory");
+  MLR_REQUIRE(extra == nullptr || merge, "a share made elsewhere joins in the merge");
   MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * D && q_stride % 8 == 0, "q_stride must cover a row and keep 16-byte alignment");
   MLR_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(key_pages) % 16 == 0 &&
                   reinterpret_cast<uintptr_t>(value_pages) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
               "operands must be 16-byte aligned");
   MLR_REQUIRE(scale > 0.f && scale < INFINITY && window >= 0 && chunk >= 0 && !(window > 0 && chunk > 0),
               "bad scale, window or chunk");
+  const int keep_partial = extra != nullptr;
   const int group = heads / kv_heads;
   const int head_tiles = (group + 15) / 16;
   MLR_REQUIRE(kv_heads * head_tiles <= 65535, "too many heads for one launch");
@@ -948,7 +985,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 #define MLR_DECODE(depth)                                                                                       \
   attn_decode_kernel<depth><<<grid, kDecodeWaves * kWave, 0, stream>>>(                                         \
       qp, q_stride, kp, vp, block_table, table_width, cu_q, context_lens, op, partial, heads, kv_heads,         \
-      head_tiles, block_size, num_pages, scale, window, chunk, part, splits, sinks)
+      head_tiles, block_size, num_pages, scale, window, chunk, part, splits, sinks, keep_partial)
   bool launched = false;
   if constexpr (kMaxDecodeDepth >= 4) {
     if (tiles_per_wave >= 4) {
@@ -966,9 +1003,9 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 #undef MLR_DECODE
   MLR_LAUNCH_CHECK();
   MLR_REQUIRE(sinks == nullptr || merge, "partitions left unmerged cannot carry sinks");
-  if (splits > 1 && merge) {
+  if ((splits > 1 || keep_partial) && merge) {
     attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
-        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks);
+        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, extra);
     MLR_LAUNCH_CHECK();
   }
   return 0;
@@ -983,7 +1020,7 @@ int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int*
   MLR_REQUIRE(entries > 0 && heads > 0 && heads <= 65535, "bad sizes");
   MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0 && chunk >= 0, "bad partitions");
   attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, context_lens,
-                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks);
+                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, nullptr);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -993,9 +1030,9 @@ int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int*
 int mlr_attention_wide_tile() { return D <= 128 ? 2 * kTileQ : 0; }
 
 // Floats of scratch mlr_attention_prefill needs when the keys of every tile are cut into
-// `splits` runs (0 for one run).
+// `splits` runs (one run writes none unless a share made elsewhere joins its softmax, see `extra`).
 int64_t mlr_attention_prefill_scratch(int num_tiles, int heads, int splits, int wide) {
-  if (splits <= 1) return 0;
+  if (splits < 1) return 0;
   return static_cast<int64_t>(num_tiles) * heads * splits * (wide ? 2 * kTileQ : kTileQ) * kPartialStride;
 }
 
@@ -1003,14 +1040,16 @@ int64_t mlr_attention_prefill_scratch(int num_tiles, int heads, int splits, int 
 // query of the tile within the entry's new tokens; 64 queries per tile, or
 // mlr_attention_wide_tile() with `wide`).  splits > 1: the keys of every tile are cut into that
 // many runs, each a workgroup of its own, and merged by a second kernel; `partial` then holds
-// mlr_attention_prefill_scratch floats.  For few tiles behind long contexts.
+// mlr_attention_prefill_scratch floats.  For few tiles behind long contexts.  `extra`: as for
+// mlr_attention_decode.
 int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages, const void* value_pages,
                           const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
                           int block_size, int num_pages, float scale, int window, int chunk, int splits,
-                          float* partial, const float* sinks, hipStream_t stream) {
+                          float* partial, const float* sinks, const float* extra, hipStream_t stream) {
   MLR_REQUIRE(splits >= 1 && splits <= 64, "splits must lie within 1..64");
-  MLR_REQUIRE(splits == 1 || partial != nullptr, "several key runs need scratch memory");
+  MLR_REQUIRE((splits == 1 && extra == nullptr) || partial != nullptr, "several key runs, or a share made elsewhere, need scratch memory");
+  const int keep_partial = extra != nullptr;
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
   MLR_REQUIRE(num_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad sizes");
   MLR_REQUIRE(kv_heads <= 65535, "too many key/value heads");  // a page's elements fit 32 bits
@@ -1053,13 +1092,13 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
           static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
-          splits > 1 ? nullptr : sinks);  \
+          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial);  \
     else                                                                                                      \
       attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
           static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
-          splits > 1 ? nullptr : sinks);  \
+          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial);  \
   } while (0)
   if constexpr (D <= 128) {
     if (wide)
@@ -1071,10 +1110,10 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   }
 #undef MLR_PREFILL
   MLR_LAUNCH_CHECK();
-  if (splits > 1) {
+  if (splits > 1 || keep_partial) {
     const int tile_q = (wide && D <= 128) ? 2 * kTileQ : kTileQ;
     attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, 0, stream>>>(
-        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q, sinks);
+        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q, sinks, extra);
     MLR_LAUNCH_CHECK();
   }
   return 0;

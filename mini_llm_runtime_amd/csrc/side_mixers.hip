@@ -165,6 +165,95 @@ __global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__
   }
 }
 
+// The pooled entries' share of a softmax that another kernel finishes: for token t (entry token_entry[t], position
+// p) and head h, over the entries j < (p - window + 1) / pool of the entry's pooled pages (none if that is not
+// positive): s_j = q . k_j * scale * log2(e), m = max s_j, l = sum 2^(s_j - m), a = sum 2^(s_j - m) v_j, left as
+// share[t, h] = [a (D floats), m, l] (m = -infinity, l = 0, a = 0 without entries).  q is bfloat16 [tokens,
+// q_stride], pages as everywhere ([page, kv head, offset, D] keys, [page, kv head, D, offset] values).  One
+// wavefront per (token, head): a lane takes every 64th entry's score, then every 64th dim of the values; 64
+// entries at a time with a running maximum.  A missing page among the entries poisons the share.
+__global__ __launch_bounds__(64) void pooled_share_kernel(const bf16* __restrict__ q, int64_t q_stride,
+                                                          const bf16* __restrict__ key_pages,
+                                                          const bf16* __restrict__ value_pages,
+                                                          const int* __restrict__ table, int table_width, int num_pages,
+                                                          const int* __restrict__ token_entry,
+                                                          const int* __restrict__ positions, float* __restrict__ share,
+                                                          int heads, int kv_heads, int D, int block_size, float scale2,
+                                                          int window, int pool) {
+  extern __shared__ float pooled_lds[];
+  float* qs = pooled_lds;      // D
+  float* ws = pooled_lds + D;  // 64 weights, then 64 page offsets (as ints)
+  int* where = reinterpret_cast<int*>(ws + 64);
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int kvh = h / (heads / kv_heads);
+  const int p = positions[t];
+  const int count = p - window + 1 > 0 ? (p - window + 1) / pool : 0;
+  float* dst = share + (t * heads + h) * (D + 2);
+  constexpr int kMaxPerLane = 4;  // head sizes up to 256
+  float acc[kMaxPerLane] = {0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  bool bad = false;
+  if (count > 0) {
+    for (int d = lane; d < D; d += 64) qs[d] = to_f32(q[t * q_stride + static_cast<int64_t>(h) * D + d]);
+    const int* row = table + static_cast<int64_t>(token_entry[t]) * table_width;
+    for (int j0 = 0; j0 < count; j0 += 64) {
+      __syncthreads();  // qs is written; the batch before is done with
+      const int j = j0 + lane;
+      float s = -INFINITY;
+      int at = -1;
+      if (j < count) {
+        const int logical = j / block_size;
+        const int page = logical < table_width ? row[logical] : -1;
+        if (page < 0 || page >= num_pages) {
+          bad = true;
+        } else {
+          at = (page * kv_heads + kvh) * block_size + (j - logical * block_size);
+          const bf16* k = key_pages + static_cast<int64_t>(at) * D;
+          float dot = 0.f;
+          for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(k[d]), dot);
+          s = dot * scale2;
+        }
+      }
+      const float m_new = fmaxf(m, wave_max(s));
+      const float keep = (m == -INFINITY) ? 0.f : exp2f(m - m_new);
+      const float w = (s == -INFINITY) ? 0.f : exp2f(s - m_new);
+      l = l * keep + wave_sum(w);
+      m = m_new;
+      ws[lane] = w;
+      where[lane] = at;
+      __syncthreads();
+      const int n = min(64, count - j0);
+#pragma unroll
+      for (int i = 0; i < kMaxPerLane; ++i) {
+        const int d = lane + 64 * i;
+        if (d >= D) break;
+        float sum = acc[i] * keep;
+        for (int u = 0; u < n; ++u) {
+          const int src = where[u];
+          if (src < 0) continue;
+          // value pages are [page, kv head, D, offset]: `src` counts (page, kv head, offset)
+          const int head_base = src / block_size;
+          const int off = src - head_base * block_size;
+          sum = fmaf(ws[u], to_f32(value_pages[(static_cast<int64_t>(head_base) * D + d) * block_size + off]), sum);
+        }
+        acc[i] = sum;
+      }
+    }
+  }
+  const bool poisoned = wave_max(bad ? 1.f : 0.f) > 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) dst[d] = poisoned ? NAN : acc[i];
+  }
+  if (lane == 0) {
+    dst[D] = poisoned ? NAN : m;
+    dst[D + 1] = l;
+  }
+}
+
 // out[t, column + head * out_dim + j] = attended[t, head * D + j] * gate[t, head] * scale for j < out_dim; gate
 // float32 [tokens, heads] (null: 1); a row of `out` is out_row elements long.
 template <typename T>
@@ -359,6 +448,25 @@ int mlr_pool_kv_write(const void* key_pages, const void* value_pages, const int*
         static_cast<const bf16*>(key_pages), static_cast<const bf16*>(value_pages), block_table, table_width, num_pages,
         token_entry, positions, pooled_slots, static_cast<bf16*>(pooled_keys), static_cast<bf16*>(pooled_values),
         pooled_pages, kv_heads, head_dim, block_size, pool);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_pooled_share(const void* q, int64_t q_stride, const void* pooled_keys, const void* pooled_values,
+                     const int* pooled_table, int table_width, int pooled_pages, const int* token_entry,
+                     const int* positions, float* share, int tokens, int heads, int kv_heads, int head_dim,
+                     int block_size, float scale, int window, int pool, hipStream_t stream) {
+  MLR_REQUIRE(q && pooled_keys && pooled_values && pooled_table && token_entry && positions && share, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && heads < 65536 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
+  MLR_REQUIRE(head_dim > 0 && head_dim <= 256, "head sizes up to 256");
+  MLR_REQUIRE(block_size > 0 && table_width > 0 && pooled_pages > 0, "pages must exist");
+  MLR_REQUIRE(q_stride >= static_cast<int64_t>(heads) * head_dim, "q_stride must cover a row");
+  MLR_REQUIRE(scale > 0.f && scale < INFINITY && window > 0 && pool > 0, "bad scale, window or run length");
+  MLR_REQUIRE(static_cast<int64_t>(pooled_pages) * kv_heads * block_size < (1ll << 31), "too many pooled slots");
+  pooled_share_kernel<<<dim3(tokens, heads), 64, (head_dim + 128) * sizeof(float), stream>>>(
+      static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(pooled_keys),
+      static_cast<const bf16*>(pooled_values), pooled_table, table_width, pooled_pages, token_entry, positions, share,
+      heads, kv_heads, head_dim, block_size, scale * 1.44269504088896340736f, window, pool);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -47,6 +47,7 @@ _SIGNATURES = {
         _I,
     ),
     "mlr_pool_kv_write": ([_VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
+    "mlr_pooled_share": ([_VP, _I64, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP], _I),
     "mlr_scale_heads": ([_VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_gla_scan": (
         [_VP, _I, _I, _I, _VP, _VP, _I, _I, _F, _VP, _VP, _I, _VP, _VP, _VP, _VP, _F, _VP, _I, _I, _I, _I, _I, _VP], _I,
@@ -95,13 +96,13 @@ _SIGNATURES = {
     "mlr_attention_wide_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP, _VP, _VP],
         _I,
     ),
     "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
     "mlr_attention_prefill_scratch": ([_I, _I, _I, _I], _I64),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP, _VP, _VP],
         _I,
     ),
 }
@@ -958,7 +959,6 @@ class HipOps:
                 raise KernelError("the pooled block table is narrower than the runs before the longest context's window")
         use_mfma = (
             kernel == "auto"
-            and pooled is None
             and self.dtype == torch.bfloat16
             and head_dim % 16 == 0
             and 16 <= head_dim <= 256
@@ -985,6 +985,17 @@ class HipOps:
             return out
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
         self._check(ctx.context_lens, "context lengths", torch.int32, (entries,))
+        share = None
+        if pooled is not None:
+            # the pooled entries' share of every token's softmax (few keys: a plain kernel); the matrix-core
+            # kernels take the window's tokens and their merge takes this share in, before the sink
+            share = self._empty((tokens, num_heads, head_dim + 2), torch.float32)
+            self._call(
+                "mlr_pooled_share", self._ptr(qkv), stride, self._ptr(pooled_keys), self._ptr(pooled_values),
+                self._ptr(pooled_table), pooled_width, pooled_pages, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
+                self._ptr(share), tokens, num_heads, num_kv_heads, head_dim, block_size, float(scale), int(window),
+                pool, self._stream(),
+            )
         if num_decode:
             span = int(plan.max_decode_context)
             if window:
@@ -1000,17 +1011,18 @@ class HipOps:
             part = -(-(-(-span // splits)) // 64) * 64
             splits = -(-span // part)
             partial = None
-            if splits > 1:
+            if splits > 1 or share is not None:
                 partial = self._empty((lib.mlr_attention_decode_scratch(entries, num_heads, splits),), torch.float32)
             leave_unmerged = (
                 defer_merge and self.tuning.fuse_merge and not num_tiles and num_decode == entries == tokens
-                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk and sinks is None
+                and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk and sinks is None and share is None
             )
             self._call(
                 "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
                 self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
-                int(window or 0), chunk, part, splits, int(not leave_unmerged), self._ptr(sinks), self._stream(), lib=lib,
+                int(window or 0), chunk, part, splits, int(not leave_unmerged), self._ptr(sinks), self._ptr(share),
+                self._stream(), lib=lib,
             )
             if leave_unmerged:
                 return PendingMerge(
@@ -1039,7 +1051,7 @@ class HipOps:
             if behind == 2 and groups < self.tuning.key_run_groups:
                 key_runs = min(8, -(-self.tuning.key_run_groups // groups))
             partial = None
-            if key_runs > 1:
+            if key_runs > 1 or share is not None:
                 partial = self._empty(
                     (lib.mlr_attention_prefill_scratch(num_tiles, num_heads, key_runs, wide),), torch.float32
                 )
@@ -1047,8 +1059,8 @@ class HipOps:
                 "mlr_attention_prefill", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
-                float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._ptr(sinks), self._stream(),
-                lib=lib,
+                float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._ptr(sinks), self._ptr(share),
+                self._stream(), lib=lib,
             )
         return out
 
