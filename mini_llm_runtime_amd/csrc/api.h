@@ -251,11 +251,15 @@ int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t 
 // Linear attention with a decay per key channel and token: decay = sigmoid(W2 low + bias)^(1 / tau) with `low` the
 // `rank` columns of `projected` from low_offset on (left in `decay` [tokens, heads * dim]); S = diag(decay) S + k v^T,
 // o = S^T (q * q_scale) per head; q, k, v are the leading columns of `projected` (float32).  State rows as for
-// mlr_retention_scan.
+// mlr_retention_scan.  `runs` (or null: every entry token by token in one wavefront per 16 value columns): scratch of
+// mlr_gla_runs(tokens, entries) * heads * dim * vdim floats, `run_decay` of mlr_gla_runs(...) * heads * dim; entries are
+// then cut into runs of 64 tokens that are walked in parallel (two walks and a carry between them).
+int mlr_gla_runs(int tokens, int entries);
 int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, const void* decay_weight,
                  const void* decay_bias, int weight_is_f32, int bias_is_f32, float tau, float* decay, float* state,
                  int state_rows, const int* read_rows, const int* write_rows, const int* cu_q, const int* q_starts,
-                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, hipStream_t stream);
+                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, float* runs,
+                 float* run_decay, hipStream_t stream);
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds

@@ -295,51 +295,88 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict_
 // lane / 16, column c = lane % 16) keeps S[d][c] for d = 4 i + g in registers; tokens go through LDS kBatch at
 // a time.  State rows as for the other recurrent kernels: read_rows[entry] (zeros when the entry starts its
 // request) to write_rows[entry]; out [tokens, heads * vdim] float32.
+//
+// Long entries are cut into runs of kGlaRun tokens (`runs` != null: blockIdx.x counts the runs of all entries, see
+// find_run), and the recurrence, which is linear in the state, is walked in three kernels:
+//   kRunSums:  every run from a zero state, no outputs: leaves U = sum_j diag(prod_{s > j} a_s) k_j v_j^T in
+//              runs[run, head] and the run's whole decay prod_s a_s in run_decay[run, head],
+//   gla_carry_kernel: per entry, run after run, S' = diag(run_decay) S + U, leaving the state BEFORE every run where
+//              its U was (the first run's: the carried state or zeros),
+//   kRunScan:  every run from its own start state, with outputs; an entry's last run stores the state.
+// Decays only ever multiply (no quotient of cumulated decays), so any decay in [0, 1] is safe.
 constexpr int kGlaBatch = 8;
+constexpr int kGlaRun = 64;
+enum GlaMode { kWholeEntries = 0, kRunSums = 1, kRunScan = 2 };
 
-template <int DPL>
+// Run `b` of all entries' runs of kGlaRun tokens: its entry, its place among the entry's runs and their number.
+__device__ inline bool find_run(int b, const int* __restrict__ cu_q, int entries, int& entry, int& index, int& count) {
+  int before = 0;
+  for (int e = 0; e < entries; ++e) {
+    const int n = (cu_q[e + 1] - cu_q[e] + kGlaRun - 1) / kGlaRun;
+    if (b < before + n) {
+      entry = e;
+      index = b - before;
+      count = n;
+      return true;
+    }
+    before += n;
+  }
+  return false;
+}
+
+template <int DPL, int MODE>
 __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ p, int width,
                                                       const float* __restrict__ decay, float* __restrict__ state,
                                                       const int* __restrict__ read_rows,
                                                       const int* __restrict__ write_rows, const int* __restrict__ cu_q,
                                                       const int* __restrict__ q_starts, float q_scale,
-                                                      float* __restrict__ out, int heads, int dim, int vdim) {
+                                                      float* __restrict__ out, int heads, int dim, int vdim,
+                                                      int entries, float* __restrict__ runs,
+                                                      float* __restrict__ run_decay) {
   __shared__ float qs[kGlaBatch][4 * DPL];
   __shared__ float ks[kGlaBatch][4 * DPL];
   __shared__ float as[kGlaBatch][4 * DPL];
   __shared__ float vs[kGlaBatch][16];
-  const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int v0 = blockIdx.z * 16;
   const int lane = threadIdx.x;
   const int g = lane / 16;
   const int c = lane % 16;
   const bool column = v0 + c < vdim;
-  const int t_first = cu_q[entry];
-  const int t_end = cu_q[entry + 1];
   const int64_t head_state = static_cast<int64_t>(dim) * vdim;
+  int entry = blockIdx.x, index = 0, count = 1;
+  if (MODE != kWholeEntries && !find_run(blockIdx.x, cu_q, entries, entry, index, count)) return;
+  int t_first = cu_q[entry];
+  int t_end = cu_q[entry + 1];
+  if (MODE != kWholeEntries) {
+    t_first += index * kGlaRun;
+    t_end = min(t_end, t_first + kGlaRun);
+  }
+  float* mine = MODE == kWholeEntries ? nullptr : runs + (static_cast<int64_t>(blockIdx.x) * heads + h) * head_state;
 
   float S[DPL];
-  const bool carried = q_starts[entry] > 0;
-  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
+  float whole[MODE == kRunSums ? DPL : 1];
+  const bool carried = MODE == kRunScan || (MODE == kWholeEntries && q_starts[entry] > 0);
+  const float* src = MODE == kRunScan ? mine : state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
     const int d = 4 * i + g;
-    S[i] = (carried && column && d < dim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+    S[i] = (MODE != kRunSums && carried && column && d < dim) ? src[static_cast<int64_t>(d) * vdim + v0 + c] : 0.f;
+    if constexpr (MODE == kRunSums) whole[i] = 1.f;
   }
   for (int tb = t_first; tb < t_end; tb += kGlaBatch) {
-    const int count = min(kGlaBatch, t_end - tb);
+    const int count_b = min(kGlaBatch, t_end - tb);
     __syncthreads();  // the batch before is done with
-    for (int idx = lane; idx < count * dim; idx += 64) {
+    for (int idx = lane; idx < count_b * dim; idx += 64) {
       const int u = idx / dim;
       const int d = idx - u * dim;
       const int64_t t = tb + u;
       const float* q = p + t * width + static_cast<int64_t>(h) * dim;
-      qs[u][d] = q[d] * q_scale;
+      if (MODE != kRunSums) qs[u][d] = q[d] * q_scale;
       ks[u][d] = q[static_cast<int64_t>(heads) * dim + d];
       as[u][d] = decay[(t * heads + h) * dim + d];
     }
-    for (int idx = lane; idx < count * 16; idx += 64) {
+    for (int idx = lane; idx < count_b * 16; idx += 64) {
       const int u = idx / 16;
       const int cc = idx - u * 16;
       vs[u][cc] = v0 + cc < vdim
@@ -347,7 +384,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                       : 0.f;
     }
     __syncthreads();
-    for (int u = 0; u < count; ++u) {
+    for (int u = 0; u < count_b; ++u) {
       const float vv = vs[u][c];
       float o = 0.f;
 #pragma unroll
@@ -355,19 +392,58 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
         const int d = 4 * i + g;
         if (d < dim) {
           S[i] = fmaf(as[u][d], S[i], ks[u][d] * vv);
-          o = fmaf(S[i], qs[u][d], o);
+          if constexpr (MODE == kRunSums)
+            whole[i] *= as[u][d];
+          else
+            o = fmaf(S[i], qs[u][d], o);
         }
       }
-      o += __shfl_xor(o, 16, kWave);
-      o += __shfl_xor(o, 32, kWave);
-      if (g == 0 && column) out[static_cast<int64_t>(tb + u) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + c] = o;
+      if (MODE != kRunSums) {
+        o += __shfl_xor(o, 16, kWave);
+        o += __shfl_xor(o, 32, kWave);
+        if (g == 0 && column) out[static_cast<int64_t>(tb + u) * heads * vdim + static_cast<int64_t>(h) * vdim + v0 + c] = o;
+      }
     }
   }
+  if constexpr (MODE == kRunSums) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = 4 * i + g;
+      if (column && d < dim) mine[static_cast<int64_t>(d) * vdim + v0 + c] = S[i];
+      if (blockIdx.z == 0 && c == 0 && d < dim) run_decay[(static_cast<int64_t>(blockIdx.x) * heads + h) * dim + d] = whole[i];
+    }
+    return;
+  }
+  if (MODE == kRunScan && index != count - 1) return;  // only an entry's last run leaves the state
   float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * head_state;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
     const int d = 4 * i + g;
     if (column && d < dim) dst[static_cast<int64_t>(d) * vdim + v0 + c] = S[i];
+  }
+}
+
+// Between the two walks over the runs (see gla_scan_kernel): a thread owns one element of one head's state and goes
+// through its entry's runs in order.  Grid (entries, heads, ceil(dim * vdim / 256)).
+__global__ __launch_bounds__(256) void gla_carry_kernel(float* __restrict__ runs, const float* __restrict__ run_decay,
+                                                        const float* __restrict__ state,
+                                                        const int* __restrict__ read_rows, const int* __restrict__ cu_q,
+                                                        const int* __restrict__ q_starts, int heads, int dim, int vdim) {
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  const int head_state = dim * vdim;
+  if (e >= head_state) return;
+  const int d = e / vdim;
+  int first = 0;  // the entry's first run among all runs
+  for (int i = 0; i < entry; ++i) first += (cu_q[i + 1] - cu_q[i] + kGlaRun - 1) / kGlaRun;
+  const int count = (cu_q[entry + 1] - cu_q[entry] + kGlaRun - 1) / kGlaRun;
+  float S = q_starts[entry] > 0 ? state[(static_cast<int64_t>(read_rows[entry]) * heads + h) * head_state + e] : 0.f;
+  for (int r = 0; r < count; ++r) {
+    float* at = runs + (static_cast<int64_t>(first + r) * heads + h) * head_state + e;
+    const float U = *at;
+    *at = S;
+    S = fmaf(run_decay[(static_cast<int64_t>(first + r) * heads + h) * dim + d], S, U);
   }
 }
 
@@ -489,10 +565,13 @@ int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t 
   return 0;
 }
 
+int mlr_gla_runs(int tokens, int entries) { return tokens / kGlaRun + entries; }
+
 int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, const void* decay_weight,
                  const void* decay_bias, int weight_is_f32, int bias_is_f32, float tau, float* decay, float* state,
                  int state_rows, const int* read_rows, const int* write_rows, const int* cu_q, const int* q_starts,
-                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, hipStream_t stream) {
+                 float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, float* runs,
+                 float* run_decay, hipStream_t stream) {
   MLR_REQUIRE(projected && decay_weight && decay && state && read_rows && write_rows && cu_q && q_starts && out,
               "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0,
@@ -505,10 +584,28 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
                                                                   decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau, decay,
                                                                   heads * dim);
   MLR_LAUNCH_CHECK();
-  dim3 grid(entries, heads, (vdim + 15) / 16);
-#define MLR_GLA(DPL)                                                                                              \
-  gla_scan_kernel<DPL><<<grid, 64, 0, stream>>>(projected, width, decay, state, read_rows, write_rows, cu_q,      \
-                                                q_starts, q_scale, out, heads, dim, vdim)
+  const dim3 whole(entries, heads, (vdim + 15) / 16);
+  const int most_runs = tokens / kGlaRun + entries;  // no fewer than the sum of the entries' runs
+  const dim3 cut(most_runs, heads, (vdim + 15) / 16);
+  const bool by_runs = runs != nullptr;
+  MLR_REQUIRE(!by_runs || run_decay != nullptr, "runs need room for their decays");
+#define MLR_GLA(DPL)                                                                                               \
+  do {                                                                                                             \
+    if (!by_runs) {                                                                                                \
+      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64, 0, stream>>>(projected, width, decay, state, read_rows,     \
+                                                                    write_rows, cu_q, q_starts, q_scale, out,      \
+                                                                    heads, dim, vdim, entries, nullptr, nullptr);  \
+    } else {                                                                                                       \
+      gla_scan_kernel<DPL, kRunSums><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
+                                                             write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
+                                                             vdim, entries, runs, run_decay);                      \
+      gla_carry_kernel<<<dim3(entries, heads, (dim * vdim + 255) / 256), 256, 0, stream>>>(                        \
+          runs, run_decay, state, read_rows, cu_q, q_starts, heads, dim, vdim);                                    \
+      gla_scan_kernel<DPL, kRunScan><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
+                                                             write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
+                                                             vdim, entries, runs, run_decay);                      \
+    }                                                                                                              \
+  } while (0)
   if (dim <= 32)
     MLR_GLA(8);
   else if (dim <= 64)

@@ -50,8 +50,9 @@ _SIGNATURES = {
     "mlr_pooled_share": ([_VP, _I64, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP], _I),
     "mlr_scale_heads": ([_VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _F, _VP], _I),
     "mlr_gla_scan": (
-        [_VP, _I, _I, _I, _VP, _VP, _I, _I, _F, _VP, _VP, _I, _VP, _VP, _VP, _VP, _F, _VP, _I, _I, _I, _I, _I, _VP], _I,
+        [_VP, _I, _I, _I, _VP, _VP, _I, _I, _F, _VP, _VP, _I, _VP, _VP, _VP, _VP, _F, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP], _I,
     ),
+    "mlr_gla_runs": ([_I, _I], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
     "mlr_scale_softcap": ([_VP, _F, _F, _I64, _VP], _I),
@@ -1442,12 +1443,15 @@ class HipOps:
         low_offset: int,
         tau: float,
         q_scale: float,
+        by_runs: Optional[bool] = None,
     ) -> torch.Tensor:
         """Linear attention with a decay per key channel and token, every entry's tokens in order: S = diag(a_t) S +
         k_t v_t^T, o_t = S^T (q_t * q_scale) per head, a_t = sigmoid(W2 low_t + bias)^(1 / tau) with low_t the columns
         low_offset .. low_offset + rank of `projected` (float32 [T, q | k | v | ...]) and W2 = decay_weight [heads *
         head_dim, rank].  State rows as for `retention_scan`.  Everything in 32-bit.  Returns o, float32 [T, heads *
-        value_dim]."""
+        value_dim].  `by_runs`: entries are cut into runs of 64 tokens that are walked in parallel, twice, with a carry
+        of the state between the walks (None: when the step has 128 tokens more than entries); else a wavefront walks
+        a whole entry token by token.  The two differ by the order of 32-bit sums only."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
         entries = ctx.num_entries
@@ -1464,13 +1468,20 @@ class HipOps:
         self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
         out = self._empty((tokens, heads * value_dim), torch.float32)
         decay = self._empty((tokens, heads * head_dim), torch.float32)
+        if by_runs is None:
+            by_runs = tokens - entries >= 128
+        runs = run_decay = None
+        if by_runs:
+            most = int(self.lib.mlr_gla_runs(tokens, entries))
+            runs = self._empty((most, heads, head_dim, value_dim), torch.float32)
+            run_decay = self._empty((most, heads, head_dim), torch.float32)
         self._call(
             "mlr_gla_scan", self._ptr(projected), width, int(low_offset), rank, self._ptr(decay_weight),
             self._ptr(decay_bias), int(decay_weight.dtype == torch.float32),
             int(decay_bias is not None and decay_bias.dtype == torch.float32), float(tau), self._ptr(decay),
             self._ptr(state), state.shape[0], self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.cu_q),
             self._ptr(ctx.q_starts), float(q_scale), self._ptr(out), entries, heads, head_dim, value_dim, tokens,
-            self._stream(),
+            self._ptr(runs), self._ptr(run_decay), self._stream(),
         )
         return out
 

@@ -353,10 +353,13 @@ def test_short_convolution_with_carried_inputs(dtype, width, taps, add):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(2, 16, 32, 5, 8.0), (3, 20, 12, 16, 1.0), (4, 64, 48, 8, 16.0), (1, 128, 16, 3, 2.0), (2, 200, 20, 1, 64.0)])
-def test_decayed_recurrence_and_its_state_rows(heads, dim, vdim, rank, tau):
-    """Three entries of unequal length (one token, a few, two chunks of 64 and a bit), two of which go on from a
-    carried state; rows of other slots stay.  Then the heads' norm with its shared weight and the gate."""
+@pytest.mark.parametrize("by_runs", [False, True], ids=["by-token", "by-run"])
+@pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(2, 16, 32, 5, 8.0), (3, 20, 12, 16, 1.0), (4, 64, 48, 8, 16.0), (1, 128, 16, 3, 2.0), (2, 200, 20, 1, 64.0), (2, 32, 64, 4, 0.05)])
+def test_decayed_recurrence_and_its_state_rows(heads, dim, vdim, rank, tau, by_runs):
+    """Three entries of unequal length (a few tokens, one, two runs of 64 and a bit), two of which go on from a
+    carried state; rows of other slots stay.  A wavefront per entry, and entries cut into runs that are walked in
+    parallel; also with a tau so small that channels forget everything within a token (decays that underflow to
+    zero).  Then the heads' norm with its shared weight and the gate."""
     ops = _ops("hip", torch.float32)
     g = torch.Generator().manual_seed(heads * dim + vdim)
     lens, starts = [5, 1, 150], [0, 40, 7]
@@ -374,6 +377,7 @@ def test_decayed_recurrence_and_its_state_rows(heads, dim, vdim, rank, tau):
     out = ops.gla_scan(
         p.cuda(), state, as_int(read), as_int(write), ctx, heads=heads, head_dim=dim, value_dim=vdim,
         decay_weight=w2.cuda(), decay_bias=bias.cuda(), low_offset=2 * qk + 2 * out_w, tau=tau, q_scale=dim**-0.5,
+        by_runs=by_runs,
     )
     for r in range(3):
         rows = p[cu[r] : cu[r + 1]].double()
