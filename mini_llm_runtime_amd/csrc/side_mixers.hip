@@ -148,18 +148,20 @@ __global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__
   const int64_t dst_base = (static_cast<int64_t>(dst_page) * kv_heads + g) * block_size * D;
   for (int i = threadIdx.x; i < D; i += 64) {
     float ks = 0.f, vs = 0.f;
+    bool gone = false;
+    // (no early exit: the loads of several positions are then on their way together)
+#pragma unroll 8
     for (int j = p - pool + 1; j <= p; ++j) {
       const int logical = j / block_size;
       const int page = logical < table_width ? table[logical] : -1;
-      if (page < 0 || page >= num_pages) {
-        ks = vs = NAN;  // a run whose tokens are gone cannot be pooled: show it
-        break;
-      }
+      const bool here = page >= 0 && page < num_pages;
+      gone = gone || !here;
       const int off = j - logical * block_size;
-      const int64_t head_base = (static_cast<int64_t>(page) * kv_heads + g) * block_size * D;
+      const int64_t head_base = (static_cast<int64_t>(here ? page : 0) * kv_heads + g) * block_size * D;
       ks += to_f32(key_pages[head_base + static_cast<int64_t>(off) * D + i]);
       vs += to_f32(value_pages[head_base + static_cast<int64_t>(i) * block_size + off]);
     }
+    if (gone) ks = vs = NAN;  // a run whose tokens are gone cannot be pooled: show it
     pooled_keys[dst_base + static_cast<int64_t>(dst_off) * D + i] = from_f32<T>(ks * inv);
     pooled_values[dst_base + static_cast<int64_t>(i) * block_size + dst_off] = from_f32<T>(vs * inv);
   }
@@ -304,8 +306,23 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict_
 //              its U was (the first run's: the carried state or zeros),
 //   kRunScan:  every run from its own start state, with outputs; an entry's last run stores the state.
 // Decays only ever multiply (no quotient of cumulated decays), so any decay in [0, 1] is safe.
-constexpr int kGlaBatch = 8;
 constexpr int kGlaRun = 64;
+// tokens that go through LDS together: every batch costs a trip to memory, but a workgroup is one wavefront and
+// a compute unit hides those trips behind its other workgroups: 12 KB each leaves room for a dozen (measured:
+// 24 KB each, six to a compute unit, is slower than batches of half the size)
+__host__ __device__ constexpr int gla_batch(int dpl) { return dpl <= 16 ? 16 : 8; }
+
+// What makes the decay of a token inside the scan kernel (entries walked whole: steps of few tokens, where a kernel
+// of its own for the decays would cost as much as the scan): see gla_decay_kernel.
+struct GlaDecayInputs {
+  int low_offset;
+  int rank;
+  const void* w2;
+  const void* bias;
+  int weight_is_f32;
+  int bias_is_f32;
+  float inv_tau;
+};
 enum GlaMode { kWholeEntries = 0, kRunSums = 1, kRunScan = 2 };
 
 // Run `b` of all entries' runs of kGlaRun tokens: its entry, its place among the entry's runs and their number.
@@ -332,7 +349,8 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       const int* __restrict__ q_starts, float q_scale,
                                                       float* __restrict__ out, int heads, int dim, int vdim,
                                                       int entries, float* __restrict__ runs,
-                                                      float* __restrict__ run_decay) {
+                                                      float* __restrict__ run_decay, GlaDecayInputs made_here) {
+  constexpr int kGlaBatch = gla_batch(DPL);
   __shared__ float qs[kGlaBatch][4 * DPL];
   __shared__ float ks[kGlaBatch][4 * DPL];
   __shared__ float as[kGlaBatch][4 * DPL];
@@ -374,7 +392,17 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
       const float* q = p + t * width + static_cast<int64_t>(h) * dim;
       if (MODE != kRunSums) qs[u][d] = q[d] * q_scale;
       ks[u][d] = q[static_cast<int64_t>(heads) * dim + d];
-      as[u][d] = decay[(t * heads + h) * dim + d];
+      if (MODE == kWholeEntries && decay == nullptr) {
+        const int ch = h * dim + d;
+        const float* low = p + t * width + made_here.low_offset;
+        float z = made_here.bias ? load_as_f32(made_here.bias, ch, made_here.bias_is_f32) : 0.f;
+        for (int r = 0; r < made_here.rank; ++r)
+          z = fmaf(load_as_f32(made_here.w2, static_cast<int64_t>(ch) * made_here.rank + r, made_here.weight_is_f32), low[r], z);
+        const float log_sigmoid = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
+        as[u][d] = expf(log_sigmoid * made_here.inv_tau);
+      } else {
+        as[u][d] = decay[(t * heads + h) * dim + d];
+      }
     }
     for (int idx = lane; idx < count_b * 16; idx += 64) {
       const int u = idx / 16;
@@ -580,30 +608,34 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
   MLR_REQUIRE(width >= 2 * heads * dim + heads * vdim, "the projected rows do not hold q, k and v");
   MLR_REQUIRE(tau > 0.f, "tau must be > 0");
   MLR_REQUIRE(dim <= 256, "heads of up to 256 dims");
-  gla_decay_kernel<<<tokens, 256, rank * sizeof(float), stream>>>(projected, width, low_offset, rank, decay_weight,
-                                                                  decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau, decay,
-                                                                  heads * dim);
-  MLR_LAUNCH_CHECK();
+  const bool by_runs = runs != nullptr;
+  const GlaDecayInputs made_here{low_offset, rank, decay_weight, decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau};
+  if (by_runs) {  // entries walked whole make their decays themselves
+    gla_decay_kernel<<<tokens, 256, rank * sizeof(float), stream>>>(projected, width, low_offset, rank, decay_weight,
+                                                                    decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau,
+                                                                    decay, heads * dim);
+    MLR_LAUNCH_CHECK();
+  }
   const dim3 whole(entries, heads, (vdim + 15) / 16);
   const int most_runs = tokens / kGlaRun + entries;  // no fewer than the sum of the entries' runs
   const dim3 cut(most_runs, heads, (vdim + 15) / 16);
-  const bool by_runs = runs != nullptr;
   MLR_REQUIRE(!by_runs || run_decay != nullptr, "runs need room for their decays");
 #define MLR_GLA(DPL)                                                                                               \
   do {                                                                                                             \
     if (!by_runs) {                                                                                                \
-      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64, 0, stream>>>(projected, width, decay, state, read_rows,     \
+      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64, 0, stream>>>(projected, width, nullptr, state, read_rows,   \
                                                                     write_rows, cu_q, q_starts, q_scale, out,      \
-                                                                    heads, dim, vdim, entries, nullptr, nullptr);  \
+                                                                    heads, dim, vdim, entries, nullptr, nullptr,   \
+                                                                    made_here);                                    \
     } else {                                                                                                       \
       gla_scan_kernel<DPL, kRunSums><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
                                                              write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
-                                                             vdim, entries, runs, run_decay);                      \
+                                                             vdim, entries, runs, run_decay, made_here);           \
       gla_carry_kernel<<<dim3(entries, heads, (dim * vdim + 255) / 256), 256, 0, stream>>>(                        \
           runs, run_decay, state, read_rows, cu_q, q_starts, heads, dim, vdim);                                    \
       gla_scan_kernel<DPL, kRunScan><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
                                                              write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
-                                                             vdim, entries, runs, run_decay);                      \
+                                                             vdim, entries, runs, run_decay, made_here);           \
     }                                                                                                              \
   } while (0)
   if (dim <= 32)

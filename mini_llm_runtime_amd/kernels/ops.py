@@ -1327,8 +1327,10 @@ class HipOps:
         head_dim: int,
         block_size: int,
         gated: bool = False,
+        projected_column: int = 0,
     ) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
-        """From the float32 sums `projected` [T, q | k | v | gate logits]: q and k each divided by the root mean
+        """From the float32 sums `projected` [T, q | k | v | gate logits] (from column `projected_column` on, when
+        the rows also hold other parts' sums): q and k each divided by the root mean
         square of their WHOLE projection and multiplied by q_norm [heads * dim] / k_norm [kv_heads * dim] (None:
         no norm), rotated (the first r dims of a head in two halves), q times head_scale[head] (float32 [heads]
         or None); k and v stored in the pages at `slot_mapping` (negative: not stored).  All in 32-bit, one
@@ -1336,7 +1338,7 @@ class HipOps:
         head size) and, if `gated`, sigmoid(gate logits) float32 [T, heads]."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
-        if width < num_heads * dim + num_kv_heads * (dim + value_dim) + (num_heads if gated else 0):
+        if projected_column < 0 or width - projected_column < num_heads * dim + num_kv_heads * (dim + value_dim) + (num_heads if gated else 0):
             raise KernelError("the projected rows are too narrow")
         weight_f32 = 0
         for w, n, name in ((q_norm, num_heads * dim, "query norm weight"), (k_norm, num_kv_heads * dim, "key norm weight")):
@@ -1360,7 +1362,7 @@ class HipOps:
         q = self._empty((tokens, num_heads * head_dim), self.dtype)
         gate = self._empty((tokens, num_heads), torch.float32) if gated else None
         self._call(
-            "mlr_qk_norm_rope_write", self._ptr(projected), width, self._ptr(q_norm), self._ptr(k_norm), weight_f32,
+            "mlr_qk_norm_rope_write", _VP(projected.data_ptr() + 4 * int(projected_column)), width, self._ptr(q_norm), self._ptr(k_norm), weight_f32,
             float(eps), self._ptr(head_scale), self._ptr(cos), self._ptr(sin), int(rotary), self._ptr(slot_mapping),
             self._ptr(key_pages), self._ptr(value_pages), self._ptr(q), self._ptr(gate), self.code, tokens, num_heads,
             num_kv_heads, dim, value_dim, head_dim, block_size, num_pages, int(bool(gated)), self._stream(),
@@ -1444,6 +1446,7 @@ class HipOps:
         tau: float,
         q_scale: float,
         by_runs: Optional[bool] = None,
+        projected_column: int = 0,
     ) -> torch.Tensor:
         """Linear attention with a decay per key channel and token, every entry's tokens in order: S = diag(a_t) S +
         k_t v_t^T, o_t = S^T (q_t * q_scale) per head, a_t = sigmoid(W2 low_t + bias)^(1 / tau) with low_t the columns
@@ -1459,7 +1462,8 @@ class HipOps:
         rank = decay_weight.shape[1]
         if decay_bias is not None:
             self._check(decay_bias, "decay bias", (torch.float32, self.dtype), (heads * head_dim,))
-        if low_offset < 0 or low_offset + rank > width or 2 * heads * head_dim + heads * value_dim > width:
+        own = width - int(projected_column)  # the rows may hold other parts' sums before this part's
+        if projected_column < 0 or low_offset < 0 or low_offset + rank > own or 2 * heads * head_dim + heads * value_dim > own:
             raise KernelError("the projected rows do not hold q, k, v and the decay's inputs")
         self._check(state, "recurrent state", torch.float32, (None, heads, head_dim, value_dim))
         self._check(read_rows, "state rows to read", torch.int32, (entries,))
@@ -1476,7 +1480,7 @@ class HipOps:
             runs = self._empty((most, heads, head_dim, value_dim), torch.float32)
             run_decay = self._empty((most, heads, head_dim), torch.float32)
         self._call(
-            "mlr_gla_scan", self._ptr(projected), width, int(low_offset), rank, self._ptr(decay_weight),
+            "mlr_gla_scan", _VP(projected.data_ptr() + 4 * int(projected_column)), width, int(low_offset), rank, self._ptr(decay_weight),
             self._ptr(decay_bias), int(decay_weight.dtype == torch.float32),
             int(decay_bias is not None and decay_bias.dtype == torch.float32), float(tau), self._ptr(decay),
             self._ptr(state), state.shape[0], self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.cu_q),

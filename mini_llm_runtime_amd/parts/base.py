@@ -39,6 +39,10 @@ class Part:
         for name, tensor in params.items():
             setattr(self, name, tensor)
 
+    def held_tensors(self) -> list:
+        """The weight tensors this part holds on the device (None where it let one go)."""
+        return [getattr(self, name) for name in self.param_specs()]
+
     def bound(self) -> None:
         """Called once every part of the model has received its parameters, nested parts before the
         parts that hold them: for what a part makes of its children's tensors."""

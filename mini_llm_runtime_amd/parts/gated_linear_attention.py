@@ -32,6 +32,8 @@ class GatedLinearAttention(Mixer):
 
     replayable = True
     open_output = True
+    open_input = True  # `activations(projected=)` takes the input product's sums from whoever made them
+    in_bias = None
 
     def __init__(
         self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay_rank: int, tau: float, norm_eps: float
@@ -78,18 +80,27 @@ class GatedLinearAttention(Mixer):
     def cache_spec(self) -> SlotStateSpec:
         return SlotStateSpec((self.num_heads, self.head_dim, self.value_dim), "float32")
 
-    def activations(self, ctx: StepContext, h, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0) -> None:
+    def activations(
+        self, ctx: StepContext, h, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0, projected=None
+    ) -> None:
+        """`projected`: (float32 sums [T, ...], first column) of h times `in_weight`, when the caller made them
+        within a larger product."""
         ops = ctx.ops
         state = ctx.state(site)
-        projected = ops.linear(h, self.in_weight, None, out_dtype=torch.float32)  # what enters the recurrence stays 32-bit
+        first = 0
+        if projected is None:
+            projected = ops.linear(h, self.in_weight, None, out_dtype=torch.float32)  # what enters the recurrence stays 32-bit
+        else:
+            projected, first = projected
         retained = ops.gla_scan(
             projected, state.tensor, state.read_rows, state.write_rows, ctx,
             heads=self.num_heads, head_dim=self.head_dim, value_dim=self.value_dim,
             decay_weight=self.decay_weight, decay_bias=self.decay_bias,
             low_offset=2 * self.qk_size + 2 * self.out_width, tau=self.tau, q_scale=self.q_scale,
+            **({"projected_column": first} if first else {}),
         )
         ops.retention_gate(
-            retained, projected, heads=self.num_heads, value_dim=self.value_dim, gate_offset=2 * self.qk_size + self.out_width,
+            retained, projected, heads=self.num_heads, value_dim=self.value_dim, gate_offset=first + 2 * self.qk_size + self.out_width,
             eps=self.norm_eps, norm_weight=self.norm_weight, scale=scale, out=out, column=column,
         )
 

@@ -132,7 +132,7 @@ class DecoderModel:
         seen: dict[int, int] = {}
         tensors = [self.embed_weight, self.head_weight, self.head_bias]
         for _, part in self.named_parts():
-            tensors.extend(getattr(part, name) for name in part.param_specs())
+            tensors.extend(part.held_tensors())
         for t in tensors:
             if t is not None:
                 seen[t.data_ptr()] = t.numel() * t.element_size()

@@ -40,6 +40,7 @@ class PooledWindowAttention(Mixer):
 
     replayable = True
     open_output = True
+    open_input = True  # `activations(projected=)` takes the input product's sums from whoever made them
 
     def __init__(
         self,
@@ -169,7 +170,11 @@ class PooledWindowAttention(Mixer):
         make = getattr(ops, "attention_plan", None)
         return make(shape) if make is not None else None
 
-    def activations(self, ctx: StepContext, h, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0) -> None:
+    def activations(
+        self, ctx: StepContext, h, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0, projected=None
+    ) -> None:
+        """`projected`: (float32 sums [T, ...], first column) of h times `in_weight` (+ `in_bias`), when the
+        caller made them within a larger product."""
         ops = ctx.ops
         if self.pool is None:
             cache, pooled = ctx.kv(site), None
@@ -178,12 +183,17 @@ class PooledWindowAttention(Mixer):
         rotation = self.position.rotation(ctx) if self.position is not None else None
         if self.position is not None and rotation is None:
             raise RuntimeError("pooled_window_attention takes position encodings that are rotations of halves")
-        projected = ops.linear(h, self.in_weight, self.in_bias, out_dtype=torch.float32)  # norm and rotation read 32-bit sums
+        first = 0
+        if projected is None:
+            projected = ops.linear(h, self.in_weight, self.in_bias, out_dtype=torch.float32)  # norm and rotation read 32-bit sums
+        else:
+            projected, first = projected
         q, gate = ops.qk_norm_rope_write(
             projected, self.q_norm_weight, self.k_norm_weight, self.norm_eps, self.head_scale, rotation,
             cache.slot_mapping, cache.key, cache.value,
             num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, dim=self.head_dim, value_dim=self.value_dim,
             head_dim=self.kernel_dim, block_size=cache.block_size, gated=self.head_gate,
+            **({"projected_column": first} if first else {}),
         )
         cache.written()
         cache.reading()

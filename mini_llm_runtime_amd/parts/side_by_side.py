@@ -22,7 +22,9 @@ class SideBySide(Mixer):
     already times its constant (in 32-bit, before their one rounding), stand side by side in one
     tensor and ONE product with the members' output matrices side by side, [Wo_a | Wo_b | ...], makes
     the sum.  That matrix is put together when the weights are bound; the members' own copies are
-    dropped.  Every member keeps its own cache: the site's cache is a composite with one member per mixer
+    dropped.  Members that take their input product's sums from outside (`open_input`: an `in_weight`
+    [rows, hidden], maybe an `in_bias`, and `activations(projected=)`) share ONE input product too: their
+    matrices one under the other, 32-bit sums, each member reading its own columns.  Every member keeps its own cache: the site's cache is a composite with one member per mixer
     that keeps one, under the mixer's name.
     """
 
@@ -45,6 +47,9 @@ class SideBySide(Mixer):
             at += member.out_width
         self._width = at
         self.o_weight: Optional[torch.Tensor] = None
+        self.in_weight: Optional[torch.Tensor] = None
+        self.in_bias: Optional[torch.Tensor] = None
+        self.in_columns: dict[str, int] = {}
 
     @property
     def out_width(self) -> int:
@@ -63,6 +68,26 @@ class SideBySide(Mixer):
         self.o_weight = torch.cat(parts, dim=1).contiguous()
         for member in self.members.values():
             member.o_weight = None
+        if len(self.members) > 1 and all(getattr(m, "open_input", False) and m.in_weight is not None for m in self.members.values()):
+            at, weights, biases = 0, [], []
+            for name, member in self.members.items():
+                self.in_columns[name] = at
+                at += member.in_weight.shape[0]
+                weights.append(member.in_weight)
+                biases.append(getattr(member, "in_bias", None))
+            self.in_weight = torch.cat(weights, dim=0).contiguous()
+            if any(b is not None for b in biases):
+                kind = next(b.dtype for b in biases if b is not None)
+                self.in_bias = torch.cat(
+                    [b.to(kind) if b is not None else w.new_zeros(w.shape[0], dtype=kind) for b, w in zip(biases, weights)]
+                ).contiguous()
+            for member in self.members.values():
+                member.in_weight = None
+                if getattr(member, "in_bias", None) is not None:
+                    member.in_bias = None
+
+    def held_tensors(self) -> list:
+        return [self.o_weight, self.in_weight, self.in_bias]
 
     def cache_spec(self) -> Any:
         specs = {name: member.cache_spec() for name, member in self.members.items()}
@@ -77,9 +102,13 @@ class SideBySide(Mixer):
         return None
 
     def activations(self, ctx: StepContext, h, site: Any, *, out: torch.Tensor, column: int, scale: float = 1.0) -> None:
+        projected = None
+        if self.in_weight is not None:
+            projected = ctx.ops.linear(h, self.in_weight, self.in_bias, out_dtype=torch.float32)
         for name, member in self.members.items():
             member.activations(
-                ctx, h, site_member(site, name), out=out, column=column + self.columns[name], scale=scale * self.scales[name]
+                ctx, h, site_member(site, name), out=out, column=column + self.columns[name], scale=scale * self.scales[name],
+                **({"projected": (projected, self.in_columns[name])} if projected is not None else {}),
             )
 
     def forward(self, ctx: StepContext, h: torch.Tensor, site: Any) -> torch.Tensor:

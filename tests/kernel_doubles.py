@@ -238,11 +238,11 @@ class TorchOps:
 
     def qk_norm_rope_write(
         self, projected, q_norm, k_norm, eps, head_scale, rotation, slot_mapping, key_pages, value_pages, *, num_heads,
-        num_kv_heads, dim, value_dim, head_dim, block_size, gated=False,
+        num_kv_heads, dim, value_dim, head_dim, block_size, gated=False, projected_column=0,
     ):
         self._count("qk_norm_rope_write")
         tokens = projected.shape[0]
-        p = projected.float()
+        p = projected.float()[:, projected_column:]
         qs, ks, vs = num_heads * dim, num_kv_heads * dim, num_kv_heads * value_dim
         q, k, v = p[:, :qs], p[:, qs : qs + ks], p[:, qs + ks : qs + ks + vs]
         if q_norm is not None:
@@ -300,11 +300,11 @@ class TorchOps:
 
     def gla_scan(
         self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, decay_weight, decay_bias,
-        low_offset, tau, q_scale,
+        low_offset, tau, q_scale, by_runs=None, projected_column=0,
     ):
         self._count("gla_scan")
         tokens = projected.shape[0]
-        p = projected.float()
+        p = projected.float()[:, projected_column:]
         qk = heads * head_dim
         q = p[:, :qk].view(tokens, heads, head_dim) * q_scale
         k = p[:, qk : 2 * qk].view(tokens, heads, head_dim)
