@@ -32,6 +32,8 @@ int mlr_rmsnorm(float* x, const void* delta, const float* partial, int slices, c
 
 // x (float32) += delta (dtype), count elements.
 int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t stream);
+// x += delta[0] + delta[1] + ... for float32 partial sums delta [slices, count], added in order.
+int mlr_add_slices(float* x, const float* delta, int slices, int64_t count, hipStream_t stream);
 
 // x (float32, in place) = x * scale, and, when cap > 0, cap * tanh(that / cap).
 int mlr_scale_softcap(float* x, float scale, float cap, int64_t count, hipStream_t stream);

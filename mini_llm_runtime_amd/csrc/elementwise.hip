@@ -160,6 +160,16 @@ __global__ __launch_bounds__(256) void add_kernel(float* __restrict__ x, const T
   if (i < count) x[i] += to_f32(delta[i]);
 }
 
+// x += delta[0] + delta[1] + ... (float32 partial sums [slices, count]), added one after the other in order
+__global__ __launch_bounds__(256) void add_slices_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                                         int slices, int64_t count) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = x[i];
+  for (int s = 0; s < slices; ++s) v += delta[static_cast<int64_t>(s) * count + i];
+  x[i] = v;
+}
+
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t* __restrict__ src,
                                                           const int* __restrict__ rows,
                                                           uint32_t* __restrict__ out, int64_t row_words,
@@ -487,6 +497,16 @@ int mlr_add(float* x, const void* delta, int dtype, int64_t count, hipStream_t s
     add_kernel<float><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, static_cast<const float*>(delta), count);
   else
     add_kernel<bf16><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, static_cast<const bf16*>(delta), count);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_add_slices(float* x, const float* delta, int slices, int64_t count, hipStream_t stream) {
+  MLR_REQUIRE(x && delta, "null pointer");
+  MLR_REQUIRE(count > 0 && slices > 0, "sizes must be > 0");
+  const int64_t blocks = (count + 255) / 256;
+  MLR_REQUIRE(blocks < (1ll << 31), "too many elements");
+  add_slices_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(x, delta, slices, count);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -123,10 +123,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
 
 // A token that completes a run of `pool` positions (pooled_slots[t] >= 0; its position p is the run's
 // last) stores the means of the run's keys and of its values, as the token pages hold them, at that
-// slot of the pooled pages (same layouts).  Sums in float32 in the order of the positions.
-// Grid (tokens, kv_heads).
+// slot of the pooled pages (same layouts).  Sums in float32: the run's positions in four quarters, each summed in
+// the order of its positions by a wavefront of its own, then the quarters in order.  Grid (tokens, kv_heads).
 template <typename T>
-__global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__ key_pages,
+__global__ __launch_bounds__(256) void pool_kv_write_kernel(const T* __restrict__ key_pages,
                                                            const T* __restrict__ value_pages,
                                                            const int* __restrict__ block_table, int table_width,
                                                            int num_pages, const int* __restrict__ token_entry,
@@ -146,12 +146,20 @@ __global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__
   if (dst_page >= pooled_pages || p - pool + 1 < 0) return;
   const float inv = 1.0f / static_cast<float>(pool);
   const int64_t dst_base = (static_cast<int64_t>(dst_page) * kv_heads + g) * block_size * D;
-  for (int i = threadIdx.x; i < D; i += 64) {
+  __shared__ float part_k[4][64], part_v[4][64];
+  __shared__ int part_gone[4];
+  const int lane = threadIdx.x % 64;
+  const int quarter = threadIdx.x / 64;
+  const int each = (pool + 3) / 4;
+  const int j_first = p - pool + 1 + quarter * each;
+  const int j_last = min(p, j_first + each - 1);
+  for (int i0 = 0; i0 < D; i0 += 64) {
+    const int i = min(i0 + lane, D - 1);
     float ks = 0.f, vs = 0.f;
     bool gone = false;
     // (no early exit: the loads of several positions are then on their way together)
 #pragma unroll 8
-    for (int j = p - pool + 1; j <= p; ++j) {
+    for (int j = j_first; j <= j_last; ++j) {
       const int logical = j / block_size;
       const int page = logical < table_width ? table[logical] : -1;
       const bool here = page >= 0 && page < num_pages;
@@ -161,9 +169,19 @@ __global__ __launch_bounds__(64) void pool_kv_write_kernel(const T* __restrict__
       ks += to_f32(key_pages[head_base + static_cast<int64_t>(off) * D + i]);
       vs += to_f32(value_pages[head_base + static_cast<int64_t>(i) * block_size + off]);
     }
-    if (gone) ks = vs = NAN;  // a run whose tokens are gone cannot be pooled: show it
-    pooled_keys[dst_base + static_cast<int64_t>(dst_off) * D + i] = from_f32<T>(ks * inv);
-    pooled_values[dst_base + static_cast<int64_t>(i) * block_size + dst_off] = from_f32<T>(vs * inv);
+    __syncthreads();  // the dims before are done with
+    part_k[quarter][lane] = ks;
+    part_v[quarter][lane] = vs;
+    if (lane == 0) part_gone[quarter] = gone;
+    __syncthreads();
+    if (quarter == 0 && i0 + lane < D) {
+      ks = ((part_k[0][lane] + part_k[1][lane]) + part_k[2][lane]) + part_k[3][lane];
+      vs = ((part_v[0][lane] + part_v[1][lane]) + part_v[2][lane]) + part_v[3][lane];
+      // a run whose tokens are gone cannot be pooled: show it
+      if (part_gone[0] || part_gone[1] || part_gone[2] || part_gone[3]) ks = vs = NAN;
+      pooled_keys[dst_base + static_cast<int64_t>(dst_off) * D + i] = from_f32<T>(ks * inv);
+      pooled_values[dst_base + static_cast<int64_t>(i) * block_size + dst_off] = from_f32<T>(vs * inv);
+    }
   }
 }
 
@@ -351,9 +369,12 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
                                                       int entries, float* __restrict__ runs,
                                                       float* __restrict__ run_decay, GlaDecayInputs made_here) {
   constexpr int kGlaBatch = gla_batch(DPL);
-  __shared__ float qs[kGlaBatch][4 * DPL];
-  __shared__ float ks[kGlaBatch][4 * DPL];
-  __shared__ float as[kGlaBatch][4 * DPL];
+  // dim d = 4 i + g lies at g * kGroup + i: a lane's DPL dims are consecutive (16-byte reads), and the four
+  // groups of a wavefront start four floats further each, in banks of their own
+  constexpr int kGroup = DPL + 4;
+  __shared__ __attribute__((aligned(16))) float qs[kGlaBatch][4 * kGroup];
+  __shared__ __attribute__((aligned(16))) float ks[kGlaBatch][4 * kGroup];
+  __shared__ __attribute__((aligned(16))) float as[kGlaBatch][4 * kGroup];
   __shared__ float vs[kGlaBatch][16];
   const int h = blockIdx.y;
   const int v0 = blockIdx.z * 16;
@@ -390,8 +411,9 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
       const int d = idx - u * dim;
       const int64_t t = tb + u;
       const float* q = p + t * width + static_cast<int64_t>(h) * dim;
-      if (MODE != kRunSums) qs[u][d] = q[d] * q_scale;
-      ks[u][d] = q[static_cast<int64_t>(heads) * dim + d];
+      const int at = (d & 3) * kGroup + (d >> 2);
+      if (MODE != kRunSums) qs[u][at] = q[d] * q_scale;
+      ks[u][at] = q[static_cast<int64_t>(heads) * dim + d];
       if (MODE == kWholeEntries && decay == nullptr) {
         const int ch = h * dim + d;
         const float* low = p + t * width + made_here.low_offset;
@@ -399,9 +421,9 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
         for (int r = 0; r < made_here.rank; ++r)
           z = fmaf(load_as_f32(made_here.w2, static_cast<int64_t>(ch) * made_here.rank + r, made_here.weight_is_f32), low[r], z);
         const float log_sigmoid = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
-        as[u][d] = expf(log_sigmoid * made_here.inv_tau);
+        as[u][at] = expf(log_sigmoid * made_here.inv_tau);
       } else {
-        as[u][d] = decay[(t * heads + h) * dim + d];
+        as[u][at] = decay[(t * heads + h) * dim + d];
       }
     }
     for (int idx = lane; idx < count_b * 16; idx += 64) {
@@ -419,11 +441,11 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
       for (int i = 0; i < DPL; ++i) {
         const int d = 4 * i + g;
         if (d < dim) {
-          S[i] = fmaf(as[u][d], S[i], ks[u][d] * vv);
+          S[i] = fmaf(as[u][g * kGroup + i], S[i], ks[u][g * kGroup + i] * vv);
           if constexpr (MODE == kRunSums)
-            whole[i] *= as[u][d];
+            whole[i] *= as[u][g * kGroup + i];
           else
-            o = fmaf(S[i], qs[u][d], o);
+            o = fmaf(S[i], qs[u][g * kGroup + i], o);
         }
       }
       if (MODE != kRunSums) {
@@ -543,12 +565,12 @@ int mlr_pool_kv_write(const void* key_pages, const void* value_pages, const int*
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
   dim3 grid(tokens, kv_heads);
   if (dtype == kF32)
-    pool_kv_write_kernel<float><<<grid, 64, 0, stream>>>(
+    pool_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
         static_cast<const float*>(key_pages), static_cast<const float*>(value_pages), block_table, table_width, num_pages,
         token_entry, positions, pooled_slots, static_cast<float*>(pooled_keys), static_cast<float*>(pooled_values),
         pooled_pages, kv_heads, head_dim, block_size, pool);
   else
-    pool_kv_write_kernel<bf16><<<grid, 64, 0, stream>>>(
+    pool_kv_write_kernel<bf16><<<grid, 256, 0, stream>>>(
         static_cast<const bf16*>(key_pages), static_cast<const bf16*>(value_pages), block_table, table_width, num_pages,
         token_entry, positions, pooled_slots, static_cast<bf16*>(pooled_keys), static_cast<bf16*>(pooled_values),
         pooled_pages, kv_heads, head_dim, block_size, pool);

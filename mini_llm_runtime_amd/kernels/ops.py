@@ -55,6 +55,7 @@ _SIGNATURES = {
     "mlr_gla_runs": ([_I, _I], _I),
     "mlr_rmsnorm": ([_VP, _VP, _VP, _I, _VP, _I, _VP, _I, _I, _I, _F, _VP], _I),
     "mlr_add": ([_VP, _VP, _I, _I64, _VP], _I),
+    "mlr_add_slices": ([_VP, _VP, _I, _I64, _VP], _I),
     "mlr_scale_softcap": ([_VP, _F, _F, _I64, _VP], _I),
     "mlr_gather_rows": ([_VP, _VP, _VP, _I, _I64, _I, _I, _VP], _I),
     "mlr_silu_mul": ([_VP, _VP, _I, _I, _I, _VP], _I),
@@ -329,9 +330,9 @@ class HipOps:
         product that has not run), in place."""
         self._check(x, "residual stream", torch.float32)
         delta = self.settle(delta)
-        if delta.dim() == x.dim() + 1:  # partial sums: one after the other, in order
-            for part in delta:
-                self.add_(x, part)
+        if delta.dim() == x.dim() + 1:  # partial sums: one after the other, in order, in one kernel
+            self._check(delta, "partial sums", torch.float32, (None, *x.shape))
+            self._call("mlr_add_slices", self._ptr(x), self._ptr(delta), delta.shape[0], x.numel(), self._stream())
             return
         self._check(delta, "residual delta", (self.dtype, torch.float32), tuple(x.shape))
         self._call("mlr_add", self._ptr(x), self._ptr(delta), _dtype_code(delta.dtype), x.numel(), self._stream())

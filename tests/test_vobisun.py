@@ -317,6 +317,23 @@ def _ctx(lens, starts):
     ), cu
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,hidden,slices", [(1, 64, 4), (8, 896, 3), (300, 70, 2)])
+def test_partial_sums_enter_the_stream_in_one_kernel(rows, hidden, slices):
+    """A mixer's output that arrives as partial sums over slices of its inner size is added to the 32-bit
+    stream slice after slice, in order (the same sums as one addition per slice)."""
+    ops = _ops("hip", torch.bfloat16)
+    g = torch.Generator().manual_seed(rows + hidden)
+    x = torch.randn(rows, hidden, generator=g)
+    parts = torch.randn(slices, rows, hidden, generator=g)
+    want = x.clone()
+    for part in parts:
+        want += part
+    stream = x.clone().cuda()
+    ops.add_(stream, parts.cuda())
+    assert torch.equal(stream.cpu(), want)
+
+
 @pytest.mark.parametrize("dtype", GPU_CASES)
 @pytest.mark.parametrize("width,taps,add", [(64, 4, True), (70, 2, True), (300, 3, False), (16, 1, True), (520, 5, True)])
 def test_short_convolution_with_carried_inputs(dtype, width, taps, add):
