@@ -313,7 +313,8 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict_
 // order; a_t [dim] from `decay` [tokens, heads * dim].  `p` [tokens, width] float32 holds q (heads * dim), k
 // (heads * dim), v (heads * vdim).  A wavefront owns 16 columns of one head's state: lane = (group of dims g =
 // lane / 16, column c = lane % 16) keeps S[d][c] for d = 4 i + g in registers; tokens go through LDS kBatch at
-// a time.  State rows as for the other recurrent kernels: read_rows[entry] (zeros when the entry starts its
+// a time, shared by the kGlaWaves wavefronts of a workgroup (64 columns: q, k and the decays are read from memory
+// once per 64 columns, not once per 16).  State rows as for the other recurrent kernels: read_rows[entry] (zeros when the entry starts its
 // request) to write_rows[entry]; out [tokens, heads * vdim] float32.
 //
 // Long entries are cut into runs of kGlaRun tokens (`runs` != null: blockIdx.x counts the runs of all entries, see
@@ -325,6 +326,7 @@ __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict_
 //   kRunScan:  every run from its own start state, with outputs; an entry's last run stores the state.
 // Decays only ever multiply (no quotient of cumulated decays), so any decay in [0, 1] is safe.
 constexpr int kGlaRun = 64;
+constexpr int kGlaWaves = 4;
 // tokens that go through LDS together: every batch costs a trip to memory, but a workgroup is one wavefront and
 // a compute unit hides those trips behind its other workgroups: 12 KB each leaves room for a dozen (measured:
 // 24 KB each, six to a compute unit, is slower than batches of half the size)
@@ -360,7 +362,7 @@ __device__ inline bool find_run(int b, const int* __restrict__ cu_q, int entries
 }
 
 template <int DPL, int MODE>
-__global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ p, int width,
+__global__ __launch_bounds__(64 * kGlaWaves) void gla_scan_kernel(const float* __restrict__ p, int width,
                                                       const float* __restrict__ decay, float* __restrict__ state,
                                                       const int* __restrict__ read_rows,
                                                       const int* __restrict__ write_rows, const int* __restrict__ cu_q,
@@ -375,10 +377,11 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   __shared__ __attribute__((aligned(16))) float qs[kGlaBatch][4 * kGroup];
   __shared__ __attribute__((aligned(16))) float ks[kGlaBatch][4 * kGroup];
   __shared__ __attribute__((aligned(16))) float as[kGlaBatch][4 * kGroup];
-  __shared__ float vs[kGlaBatch][16];
+  __shared__ float vs[kGlaBatch][16 * kGlaWaves];
   const int h = blockIdx.y;
-  const int v0 = blockIdx.z * 16;
-  const int lane = threadIdx.x;
+  const int wave = threadIdx.x / 64;
+  const int v0 = (blockIdx.z * kGlaWaves + wave) * 16;
+  const int lane = threadIdx.x % 64;
   const int g = lane / 16;
   const int c = lane % 16;
   const bool column = v0 + c < vdim;
@@ -406,7 +409,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
   for (int tb = t_first; tb < t_end; tb += kGlaBatch) {
     const int count_b = min(kGlaBatch, t_end - tb);
     __syncthreads();  // the batch before is done with
-    for (int idx = lane; idx < count_b * dim; idx += 64) {
+    for (int idx = threadIdx.x; idx < count_b * dim; idx += 64 * kGlaWaves) {
       const int u = idx / dim;
       const int d = idx - u * dim;
       const int64_t t = tb + u;
@@ -426,16 +429,15 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
         as[u][at] = decay[(t * heads + h) * dim + d];
       }
     }
-    for (int idx = lane; idx < count_b * 16; idx += 64) {
-      const int u = idx / 16;
-      const int cc = idx - u * 16;
-      vs[u][cc] = v0 + cc < vdim
-                      ? p[static_cast<int64_t>(tb + u) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v0 + cc]
-                      : 0.f;
+    for (int idx = threadIdx.x; idx < count_b * 16 * kGlaWaves; idx += 64 * kGlaWaves) {
+      const int u = idx / (16 * kGlaWaves);
+      const int cc = idx - u * (16 * kGlaWaves);
+      const int v = blockIdx.z * 16 * kGlaWaves + cc;
+      vs[u][cc] = v < vdim ? p[static_cast<int64_t>(tb + u) * width + 2ll * heads * dim + static_cast<int64_t>(h) * vdim + v] : 0.f;
     }
     __syncthreads();
     for (int u = 0; u < count_b; ++u) {
-      const float vv = vs[u][c];
+      const float vv = vs[u][wave * 16 + c];
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
@@ -460,7 +462,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(const float* __restrict__ 
     for (int i = 0; i < DPL; ++i) {
       const int d = 4 * i + g;
       if (column && d < dim) mine[static_cast<int64_t>(d) * vdim + v0 + c] = S[i];
-      if (blockIdx.z == 0 && c == 0 && d < dim) run_decay[(static_cast<int64_t>(blockIdx.x) * heads + h) * dim + d] = whole[i];
+      if (blockIdx.z == 0 && wave == 0 && c == 0 && d < dim) run_decay[(static_cast<int64_t>(blockIdx.x) * heads + h) * dim + d] = whole[i];
     }
     return;
   }
@@ -638,24 +640,24 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
                                                                     decay, heads * dim);
     MLR_LAUNCH_CHECK();
   }
-  const dim3 whole(entries, heads, (vdim + 15) / 16);
+  const dim3 whole(entries, heads, (vdim + 16 * kGlaWaves - 1) / (16 * kGlaWaves));
   const int most_runs = tokens / kGlaRun + entries;  // no fewer than the sum of the entries' runs
-  const dim3 cut(most_runs, heads, (vdim + 15) / 16);
+  const dim3 cut(most_runs, heads, (vdim + 16 * kGlaWaves - 1) / (16 * kGlaWaves));
   MLR_REQUIRE(!by_runs || run_decay != nullptr, "runs need room for their decays");
 #define MLR_GLA(DPL)                                                                                               \
   do {                                                                                                             \
     if (!by_runs) {                                                                                                \
-      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64, 0, stream>>>(projected, width, nullptr, state, read_rows,   \
+      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64 * kGlaWaves, 0, stream>>>(projected, width, nullptr, state, read_rows,   \
                                                                     write_rows, cu_q, q_starts, q_scale, out,      \
                                                                     heads, dim, vdim, entries, nullptr, nullptr,   \
                                                                     made_here);                                    \
     } else {                                                                                                       \
-      gla_scan_kernel<DPL, kRunSums><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
+      gla_scan_kernel<DPL, kRunSums><<<cut, 64 * kGlaWaves, 0, stream>>>(projected, width, decay, state, read_rows,            \
                                                              write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
                                                              vdim, entries, runs, run_decay, made_here);           \
       gla_carry_kernel<<<dim3(entries, heads, (dim * vdim + 255) / 256), 256, 0, stream>>>(                        \
           runs, run_decay, state, read_rows, cu_q, q_starts, heads, dim, vdim);                                    \
-      gla_scan_kernel<DPL, kRunScan><<<cut, 64, 0, stream>>>(projected, width, decay, state, read_rows,            \
+      gla_scan_kernel<DPL, kRunScan><<<cut, 64 * kGlaWaves, 0, stream>>>(projected, width, decay, state, read_rows,            \
                                                              write_rows, cu_q, q_starts, q_scale, out, heads, dim, \
                                                              vdim, entries, runs, run_decay, made_here);           \
     }                                                                                                              \
