@@ -395,6 +395,13 @@ __global__ __launch_bounds__(64 * kGlaWaves) void gla_scan_kernel(const float* _
     t_end = min(t_end, t_first + kGlaRun);
   }
   float* mine = MODE == kWholeEntries ? nullptr : runs + (static_cast<int64_t>(blockIdx.x) * heads + h) * head_state;
+  // dims beyond `dim` read zeros (a decay of 0 on a state of 0), so that the walk below needs no condition per dim:
+  // a condition there makes every LDS read wait for the one before
+  for (int idx = threadIdx.x; idx < kGlaBatch * 4 * kGroup; idx += 64 * kGlaWaves) {
+    (&qs[0][0])[idx] = 0.f;
+    (&ks[0][0])[idx] = 0.f;
+    (&as[0][0])[idx] = 0.f;
+  }
 
   float S[DPL];
   float whole[MODE == kRunSums ? DPL : 1];
@@ -441,14 +448,12 @@ __global__ __launch_bounds__(64 * kGlaWaves) void gla_scan_kernel(const float* _
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
-        const int d = 4 * i + g;
-        if (d < dim) {
-          S[i] = fmaf(as[u][g * kGroup + i], S[i], ks[u][g * kGroup + i] * vv);
-          if constexpr (MODE == kRunSums)
-            whole[i] *= as[u][g * kGroup + i];
-          else
-            o = fmaf(S[i], qs[u][g * kGroup + i], o);
-        }
+        const float a = as[u][g * kGroup + i];
+        S[i] = fmaf(a, S[i], ks[u][g * kGroup + i] * vv);
+        if constexpr (MODE == kRunSums)
+          whole[i] *= a;
+        else
+          o = fmaf(S[i], qs[u][g * kGroup + i], o);
       }
       if (MODE != kRunSums) {
         o += __shfl_xor(o, 16, kWave);
