@@ -232,7 +232,19 @@ __global__ __launch_bounds__(64) void pooled_share_kernel(const bf16* __restrict
           at = (page * kv_heads + kvh) * block_size + (j - logical * block_size);
           const bf16* k = key_pages + static_cast<int64_t>(at) * D;
           float dot = 0.f;
-          for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(k[d]), dot);
+          if (D % 8 == 0) {  // rows of whole 16-byte pieces (pages are 16-byte aligned)
+            for (int d = 0; d < D; d += 8) {
+              const uint4 piece = *reinterpret_cast<const uint4*>(k + d);
+              const uint32_t words[4] = {piece.x, piece.y, piece.z, piece.w};
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                dot = fmaf(qs[d + 2 * j], __uint_as_float(words[j] << 16), dot);
+                dot = fmaf(qs[d + 2 * j + 1], __uint_as_float(words[j] & 0xffff0000u), dot);
+              }
+            }
+          } else {
+            for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(k[d]), dot);
+          }
           s = dot * scale2;
         }
       }
@@ -333,7 +345,9 @@ constexpr int kGlaWaves = 4;
 __host__ __device__ constexpr int gla_batch(int dpl) { return dpl <= 16 ? 16 : 8; }
 
 // What makes the decay of a token inside the scan kernel (entries walked whole: steps of few tokens, where a kernel
-// of its own for the decays would cost as much as the scan): see gla_decay_kernel.
+// of its own for the decays would cost as much as the scan; inside the walks over runs it was measured slower than
+// that kernel: it holds up a workgroup's four wavefronts and is made again for every 64 value columns): see
+// gla_decay_kernel.
 struct GlaDecayInputs {
   int low_offset;
   int rank;
@@ -424,7 +438,7 @@ __global__ __launch_bounds__(64 * kGlaWaves) void gla_scan_kernel(const float* _
       const int at = (d & 3) * kGroup + (d >> 2);
       if (MODE != kRunSums) qs[u][at] = q[d] * q_scale;
       ks[u][at] = q[static_cast<int64_t>(heads) * dim + d];
-      if (MODE == kWholeEntries && decay == nullptr) {
+      if (MODE == kWholeEntries) {
         const int ch = h * dim + d;
         const float* low = p + t * width + made_here.low_offset;
         float z = made_here.bias ? load_as_f32(made_here.bias, ch, made_here.bias_is_f32) : 0.f;
@@ -652,7 +666,7 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
 #define MLR_GLA(DPL)                                                                                               \
   do {                                                                                                             \
     if (!by_runs) {                                                                                                \
-      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64 * kGlaWaves, 0, stream>>>(projected, width, nullptr, state, read_rows,   \
+      gla_scan_kernel<DPL, kWholeEntries><<<whole, 64 * kGlaWaves, 0, stream>>>(projected, width, decay, state, read_rows,     \
                                                                     write_rows, cu_q, q_starts, q_scale, out,      \
                                                                     heads, dim, vdim, entries, nullptr, nullptr,   \
                                                                     made_here);                                    \
