@@ -58,10 +58,10 @@ class VobisunRotary:
                 raise ConfigError(f"{where}: 'scaling' must be an object or null")
             require_keys(scaling, ("factor",), where + ".scaling")
             factor = positive_float(scaling, "factor")
-        out = cls(base=positive_float(data, "base"), dims=positive_int(data, "dims"), factor=factor)
-        if out.dims % 2:
-            raise ConfigError(f"{where}: dims must be even")
-        return out
+        dims = data["dims"]
+        if isinstance(dims, bool) or not isinstance(dims, int) or dims < 0 or dims % 2:
+            raise ConfigError(f"{where}: dims must be an even integer >= 0 (0: nothing turns), found {dims!r}")
+        return cls(base=positive_float(data, "base"), dims=int(dims), factor=factor)
 
     def to_dict(self) -> dict[str, Any]:
         out: dict[str, Any] = {"base": self.base, "dims": self.dims}

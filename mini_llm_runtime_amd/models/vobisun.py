@@ -47,7 +47,8 @@ def vobisun_spec(config: VobisunConfig) -> ModelSpec:
             "pooled_window_attention",
             {
                 "hidden_size": width, "num_heads": a.heads, "num_kv_heads": a.kv_heads, "head_dim": a.dim,
-                "value_dim": a.vdim, "window": a.window, "pool": a.pool, "scale": a.scale, "position": rotary,
+                "value_dim": a.vdim, "window": a.window, "pool": a.pool, "scale": a.scale,
+                "position": rotary if a.rot.dims > 0 else None,  # no dims turn: no position encoding at all
                 "qkv_bias": True, "qk_norm": True, "norm_eps": eps, "temperature": True, "sink": True, "head_gate": True,
             },
         )

@@ -97,11 +97,12 @@ CONFIGS = {
         _layer(_left(4, 1, 32, 48, 300, 8, 16, 4.0, 0.2), _right(2, 64, 64, 64.0), 96),
         _layer(_left(2, 2, 64, 32, 40, 5, 64, None, 0.15), _right(4, 32, 16, 8.0), None),
     ]),
-    # values that could hide a fault by being 1: one tap (no carried inputs), a window of one token, pooled
-    # blocks of one token (every older token is its own block), one head everywhere, a loop that runs once
+    # values that could hide a fault by being 1 or 0: one tap (no carried inputs), a window of one token, pooled
+    # blocks of one token (every older token is its own block), one head, a loop that runs once, heads of which
+    # no dims turn
     "E": _model(96, 48, 1e-6, 1.0, 1, [
         _layer(_left(1, 1, 16, 16, 1, 1, 2, 1.0, 0.3), _right(1, 16, 16, 1.0), 40),
-        _layer(_left(2, 2, 8, 8, 3, 1, 8, None, 0.4), _right(2, 8, 8, 5.0), None),
+        _layer(_left(2, 2, 8, 8, 3, 1, 0, None, 0.4), _right(2, 8, 8, 5.0), None),  # no dims turn
     ], loop=(0, 2, 1)),
     # one half of the mixer at a time: what it does is not blurred by the other
     "L": _model(128, 64, 1e-6, 3.0, 3, [_layer(_left(4, 2, 16, 32, 12, 4, 12, 2.0, 0.3), _right(1, 8, 8, 2.0), None, 1.0, 0.0)]),
@@ -618,6 +619,46 @@ def test_replayed_steps_equal_plain_steps(tmp_path, dtype):
     assert plain_steps.keys() == replayed.keys()
     for key in plain_steps:
         assert torch.equal(plain_steps[key], replayed[key]), key
+
+
+@pytest.mark.gpu
+def test_long_requests_in_bfloat16_against_the_float32_engine(tmp_path):
+    """Requests of thousands of tokens in portions of 512 beside a decoding request: portions sit behind thousands
+    of cached tokens (the prompt kernel's long-prefix levels and key runs, whose merge also takes in the pooled
+    entries' share), a window of 1,500 tokens spans a hundred pages, a hundred pooled blocks.  The plain
+    implementation is too slow at this length; the float32 engine, which it checks at shorter lengths and which
+    runs other kernels throughout, stands in for it."""
+    cfg = _model(160, 128, 1e-5, 4.0, 3, [
+        _layer(_left(4, 2, 64, 64, 1500, 32, 32, 4.0, 0.12), _right(2, 64, 64, 32.0), 128),
+        _layer(_left(2, 1, 32, 48, 700, 64, 16, None, 0.2), _right(2, 32, 32, 8.0), None),
+    ], loop=(1, 2, 2))
+    weights = make_weights(cfg, 17)
+    folder = write_model(tmp_path, "long", cfg, weights)
+    requests = {"a": random_tokens(4700, 160, 1), "b": random_tokens(2300, 160, 2)}
+    want = {"a": [0, 511, 512, 1499, 1500, 1531, 1532, 2047, 2048, 3000, 4095, 4096, 4699], "b": [0, 699, 700, 763, 764, 2299]}
+    steps, fed = [], {"a": 0, "b": 0}
+    while any(fed[r] < len(requests[r]) for r in requests):
+        entries, end = [], []
+        for rid, toks in requests.items():
+            if fed[rid] >= len(toks):
+                continue
+            n = min(512 if rid == "a" else (2296 if fed[rid] == 0 else 1), len(toks) - fed[rid])
+            entries.append({"id": rid, "tokens": toks[fed[rid] : fed[rid] + n], "want": [w - fed[rid] for w in want[rid] if fed[rid] <= w < fed[rid] + n]})
+            fed[rid] += n
+            if fed[rid] == len(toks):
+                end.append(rid)
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    results = {}
+    for dtype, plan in ((torch.float32, schedules.whole({r: t for r, t in requests.items()})), (torch.bfloat16, steps)):
+        _, _, cache, runner = make_runner(folder, _ops("hip", dtype), block_size=16, num_blocks=2 * (7000 // 16 + 4), max_requests=2)
+        cache.poison()
+        results[dtype] = schedules.run_schedule(runner, cache, plan)
+        cache.check_invariants()
+    for rid in requests:
+        for pos in want[rid]:
+            ref, got = results[torch.float32][(rid, pos)].double(), results[torch.bfloat16][(rid, pos)].double()
+            rel = float((got - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt())
+            assert rel < 6e-2, (rid, pos, rel)
 
 
 # ---- generation through the engine ------------------------------------------------------------------------
