@@ -305,19 +305,38 @@ __global__ __launch_bounds__(256) void scale_heads_kernel(const T* __restrict__ 
 // decay[t, c] = sigmoid(z)^(1 / tau), z = sum_r w2[c, r] * low[t, r] + bias[c]: `low` are `rank` columns of
 // the projected rows p (float32) from column low_offset on, w2 [channels, rank], all sums in float32.
 // log sigmoid(z) = -softplus(-z), taken on the side where the exponential is small.
+constexpr int kDecayTokens = 8;
+
 __global__ __launch_bounds__(256) void gla_decay_kernel(const float* __restrict__ p, int width, int low_offset, int rank,
                                                         const void* __restrict__ w2, const void* __restrict__ bias,
                                                         int weight_is_f32, int bias_is_f32, float inv_tau,
-                                                        float* __restrict__ decay, int channels) {
-  extern __shared__ float low[];
-  const int64_t t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += 256) low[r] = p[t * width + low_offset + r];
+                                                        float* __restrict__ decay, int channels, int tokens) {
+  // a workgroup takes kDecayTokens tokens, so that a row of w2 is read once for all of them
+  extern __shared__ float low[];  // [kDecayTokens][rank]
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kDecayTokens;
+  const int count = static_cast<int>(min(static_cast<int64_t>(kDecayTokens), tokens - t0));
+  for (int idx = threadIdx.x; idx < count * rank; idx += 256) {
+    const int u = idx / rank;
+    const int r = idx - u * rank;
+    low[idx] = p[(t0 + u) * width + low_offset + r];
+  }
   __syncthreads();
   for (int c = threadIdx.x; c < channels; c += 256) {
-    float z = bias ? load_as_f32(bias, c, bias_is_f32) : 0.f;
-    for (int r = 0; r < rank; ++r) z = fmaf(load_as_f32(w2, static_cast<int64_t>(c) * rank + r, weight_is_f32), low[r], z);
-    const float log_sigmoid = z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z));
-    decay[t * channels + c] = expf(log_sigmoid * inv_tau);
+    float z[kDecayTokens];
+    const float b = bias ? load_as_f32(bias, c, bias_is_f32) : 0.f;
+#pragma unroll
+    for (int u = 0; u < kDecayTokens; ++u) z[u] = b;
+    for (int r = 0; r < rank; ++r) {
+      const float w = load_as_f32(w2, static_cast<int64_t>(c) * rank + r, weight_is_f32);
+#pragma unroll
+      for (int u = 0; u < kDecayTokens; ++u) z[u] = fmaf(w, low[min(u, count - 1) * rank + r], z[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kDecayTokens; ++u) {
+      if (u >= count) break;
+      const float log_sigmoid = z[u] >= 0.f ? -log1pf(expf(-z[u])) : z[u] - log1pf(expf(z[u]));
+      decay[(t0 + u) * channels + c] = expf(log_sigmoid * inv_tau);
+    }
   }
 }
 
@@ -647,16 +666,16 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
               "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0,
               "sizes must be > 0");
-  MLR_REQUIRE(rank > 0 && rank <= 4096 && low_offset >= 0 && width >= low_offset + rank, "the projected rows do not hold the decay's inputs");
+  MLR_REQUIRE(rank > 0 && rank <= 2048 && low_offset >= 0 && width >= low_offset + rank, "the projected rows do not hold the decay's inputs");
   MLR_REQUIRE(width >= 2 * heads * dim + heads * vdim, "the projected rows do not hold q, k and v");
   MLR_REQUIRE(tau > 0.f, "tau must be > 0");
   MLR_REQUIRE(dim <= 256, "heads of up to 256 dims");
   const bool by_runs = runs != nullptr;
   const GlaDecayInputs made_here{low_offset, rank, decay_weight, decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau};
   if (by_runs) {  // entries walked whole make their decays themselves
-    gla_decay_kernel<<<tokens, 256, rank * sizeof(float), stream>>>(projected, width, low_offset, rank, decay_weight,
-                                                                    decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau,
-                                                                    decay, heads * dim);
+    gla_decay_kernel<<<(tokens + kDecayTokens - 1) / kDecayTokens, 256, kDecayTokens * rank * sizeof(float), stream>>>(
+        projected, width, low_offset, rank, decay_weight, decay_bias, weight_is_f32, bias_is_f32, 1.0f / tau, decay,
+        heads * dim, tokens);
     MLR_LAUNCH_CHECK();
   }
   const dim3 whole(entries, heads, (vdim + 16 * kGlaWaves - 1) / (16 * kGlaWaves));
