@@ -251,7 +251,7 @@ int mlr_scale_heads(const void* attended, const float* gate, void* out, int64_t 
                     int head_dim, int out_dim, float scale, hipStream_t stream);
 
 // Linear attention with a decay per key channel and token: decay = sigmoid(W2 low + bias)^(1 / tau) with `low` the
-// `rank` columns of `projected` from low_offset on (left in `decay` [tokens, heads * dim]); S = diag(decay) S + k v^T,
+// `rank` columns of `projected` from low_offset on (with `runs`, left in `decay` [tokens, heads * dim]); S = diag(decay) S + k v^T,
 // o = S^T (q * q_scale) per head; q, k, v are the leading columns of `projected` (float32).  State rows as for
 // mlr_retention_scan.  `runs` (or null: every entry token by token in one wavefront per 16 value columns): scratch of
 // mlr_gla_runs(tokens, entries) * heads * dim * vdim floats, `run_decay` of mlr_gla_runs(...) * heads * dim; entries are

@@ -662,8 +662,8 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
                  int state_rows, const int* read_rows, const int* write_rows, const int* cu_q, const int* q_starts,
                  float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, float* runs,
                  float* run_decay, hipStream_t stream) {
-  MLR_REQUIRE(projected && decay_weight && decay && state && read_rows && write_rows && cu_q && q_starts && out,
-              "null pointer");
+  MLR_REQUIRE(projected && decay_weight && state && read_rows && write_rows && cu_q && q_starts && out, "null pointer");
+  MLR_REQUIRE(runs == nullptr || decay != nullptr, "runs need room for the tokens' decays");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0,
               "sizes must be > 0");
   MLR_REQUIRE(rank > 0 && rank <= 2048 && low_offset >= 0 && width >= low_offset + rank, "the projected rows do not hold the decay's inputs");

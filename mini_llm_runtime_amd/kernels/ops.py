@@ -1472,11 +1472,11 @@ class HipOps:
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
         self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
         out = self._empty((tokens, heads * value_dim), torch.float32)
-        decay = self._empty((tokens, heads * head_dim), torch.float32)
         if by_runs is None:
             by_runs = tokens - entries >= 128
-        runs = run_decay = None
+        decay = runs = run_decay = None
         if by_runs:
+            decay = self._empty((tokens, heads * head_dim), torch.float32)
             most = int(self.lib.mlr_gla_runs(tokens, entries))
             runs = self._empty((most, heads, head_dim, value_dim), torch.float32)
             run_decay = self._empty((most, heads, head_dim), torch.float32)

@@ -12,6 +12,28 @@ from __future__ import annotations
 import torch
 
 F64 = torch.float64
+_ROUND = False
+
+
+class rounded:
+    """Within this context every product's input is rounded to bfloat16 first (the weights are bfloat16 anyway):
+    what rounding alone does to a row, as a yardstick for rows on which the engine's bfloat16 and the exact
+    result differ much (a head's norm of a near-zero output is a sign function)."""
+
+    def __enter__(self):
+        global _ROUND
+        self.before, _ROUND = _ROUND, True
+
+    def __exit__(self, *exc):
+        global _ROUND
+        _ROUND = self.before
+
+
+def _mm(x, w):
+    """x times w transposed."""
+    if _ROUND:
+        x = x.to(torch.bfloat16).to(F64)
+    return x @ w.T
 
 
 def rms_norm(x, weight, eps):
@@ -79,9 +101,9 @@ def left_mixer(h, w, p, cfg, eps, positions):
     partial rotation, window with pooled blocks, sink, a gate per head, output projection."""
     H, G, d, dv = cfg["heads"], cfg["kv_heads"], cfg["dim"], cfg["vdim"]
     T = h.shape[0]
-    q = h @ w[p + "q"].T + w[p + "q.b"]
-    k = h @ w[p + "k"].T + w[p + "k.b"]
-    v = h @ w[p + "v"].T + w[p + "v.b"]
+    q = _mm(h, w[p + "q"]) + w[p + "q.b"]
+    k = _mm(h, w[p + "k"]) + w[p + "k.b"]
+    v = _mm(h, w[p + "v"]) + w[p + "v.b"]
     q = rms_norm(q, w[p + "q.norm"], eps).view(T, H, d)
     k = rms_norm(k, w[p + "k.norm"], eps).view(T, G, d)
     v = v.view(T, G, dv)
@@ -93,9 +115,9 @@ def left_mixer(h, w, p, cfg, eps, positions):
         q, k, v, window=cfg["mask"]["size"], pool=cfg["mask"]["pool"], scale=cfg["scale"],
         temp=w[p + "temp"], sink=w[p + "sink"],
     )
-    gate = torch.sigmoid(h @ w[p + "g"].T)  # [T, H]
+    gate = torch.sigmoid(_mm(h, w[p + "g"]))  # [T, H]
     a = a * gate[:, :, None]
-    return a.reshape(T, H * dv) @ w[p + "o"].T
+    return _mm(a.reshape(T, H * dv), w[p + "o"])
 
 
 def gated_linear_attention(q, k, v, alpha):
@@ -115,20 +137,20 @@ def right_mixer(h, w, p, cfg, eps):
     per head with one shared weight, a silu gate, output projection."""
     H, d, dv, tau = cfg["heads"], cfg["dim"], cfg["vdim"], cfg["tau"]
     T = h.shape[0]
-    q = (h @ w[p + "q"].T * d ** -0.5).view(T, H, d)
-    k = (h @ w[p + "k"].T).view(T, H, d)
-    v = (h @ w[p + "v"].T).view(T, H, dv)
-    z = (h @ w[p + "a1"].T) @ w[p + "a2"].T + w[p + "a2.b"]
+    q = (_mm(h, w[p + "q"]) * d ** -0.5).view(T, H, d)
+    k = (_mm(h, w[p + "k"])).view(T, H, d)
+    v = (_mm(h, w[p + "v"])).view(T, H, dv)
+    z = _mm(h, w[p + "a1"]) @ w[p + "a2"].T + w[p + "a2.b"]  # the second product stays exact: it enters the recurrence
     alpha = torch.sigmoid(z).pow(1.0 / tau).view(T, H, d)
     o = gated_linear_attention(q, k, v, alpha)
     o = rms_norm(o, w[p + "norm"], eps).reshape(T, H * dv)
-    g = h @ w[p + "g"].T
-    return (o * g * torch.sigmoid(g)) @ w[p + "o"].T
+    g = _mm(h, w[p + "g"])
+    return _mm(o * g * torch.sigmoid(g), w[p + "o"])
 
 
 def dense_feed_forward(h, w, p):
-    g = h @ w[p + "gate"].T
-    return (g * torch.sigmoid(g) * (h @ w[p + "up"].T)) @ w[p + "down"].T
+    g = _mm(h, w[p + "gate"])
+    return _mm(g * torch.sigmoid(g) * _mm(h, w[p + "up"]), w[p + "down"])
 
 
 def layer(x, w, i, cfg, config, positions):
@@ -165,6 +187,6 @@ def forward(config, weights, tokens, return_layers=False):
     for i in layer_runs(config):
         x = layer(x, w, i, config["layers"][i], config, positions)
         streams.append(x)
-    logits = rms_norm(x, w["final.norm"], config["norm"]["eps"]) @ w["head"].T
+    logits = _mm(rms_norm(x, w["final.norm"], config["norm"]["eps"]), w["head"])
     return (logits, torch.stack(streams)) if return_layers else logits
 

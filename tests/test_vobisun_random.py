@@ -3,7 +3,10 @@ a drawn schedule and page size, the engine against the plain implementation.  A 
 nobody has looked at must run without a change of code; this is the nearest a test gets.
 
 The bounds are those of `test_vobisun._compare`, the float32 one a little wider (drawn models of many layer
-runs add up more 32-bit roundings than the chosen ones)."""
+runs add up more 32-bit roundings than the chosen ones).  108 more from the same generator ran once on the GPU in both
+dtypes: float32 passed all; bfloat16 missed the bound in seven, each time from a request's first token on, where a
+recurrent head's q . k was within a rounding of zero (`test_vobisun._first_token_is_a_coin_flip`; the stand-in on the
+CPU, which shares no kernel, gave the same rows to three digits)."""
 
 from __future__ import annotations
 
@@ -83,6 +86,9 @@ def test_drawn_configuration_on_the_stand_in(tmp_path, seed):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("seed", range(32))
-def test_drawn_configuration(tmp_path, seed):
-    _run(tmp_path, seed, "hip", torch.float32 if seed % 2 else torch.bfloat16)
+def test_drawn_configuration(tmp_path, seed, dtype):
+    """Both dtypes on every drawn model: requests whose first token is a coin flip are left out in bfloat16 (see
+    `_compare`), never in float32."""
+    _run(tmp_path, seed, "hip", dtype)
