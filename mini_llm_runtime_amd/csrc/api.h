@@ -169,7 +169,7 @@ int mlr_paged_attention_simple(const void* q, int64_t q_stride, const void* key_
                                int block_size, int num_pages, float scale, int window, int chunk,
                                const float* sinks, const void* pooled_keys, const void* pooled_values,
                                const int* pooled_table, int pooled_width, int pooled_pages, int pool,
-                               hipStream_t stream);
+                               const float* score_bias, hipStream_t stream);
 
 // x (float32 [rows, hidden], in place) += weight * y * rsqrt(mean(y^2) + eps), y [rows, hidden] float32
 // or `dtype`, or `slices` float32 partial sums [slices, rows, hidden].  Then mode 1: out = next_weight * x *
@@ -188,7 +188,7 @@ int mlr_latent_prepare(const float* projected, int width, void* q_plain, void* q
                        const float* sin, int rotary_dims, const void* norm_weight, int weight_is_f32, float eps,
                        const int* slots, void* key_pages, void* value_pages, int dtype, int tokens, int heads, int dim,
                        int rot, int rank, int kernel_dim, int block_size, int num_pages, int own_cache, int gated,
-                       hipStream_t stream);
+                       const float* queries, int q_width, hipStream_t stream);
 
 // out[t * out_row + h * out_stride + j] = row_scale[t, h] * sum_i x[t * in_row + h * in_stride + i] * w[h, j, i].
 int mlr_heads_linear(const void* x, int64_t in_row, int in_stride, const void* w, void* out, int64_t out_row,
@@ -210,7 +210,7 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
 // gate_offset + h * vdim + :]) * out_scale; norm_weight [vdim] is shared by the heads (null: none).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
                        int tokens, int heads, int vdim, float eps, const void* norm_weight, int weight_is_f32,
-                       float out_scale, int64_t out_row, hipStream_t stream);
+                       float out_scale, int64_t out_row, int weight_per_head, int gate_kind, hipStream_t stream);
 
 // out[t] = (add_input ? h[t] : 0) + a causal convolution over the entry's inputs of `taps` taps per channel (weight
 // [width, taps], the last tap on the token itself); the taps - 1 inputs before a step are carried in `state`
@@ -263,6 +263,23 @@ int mlr_gla_scan(const float* projected, int width, int low_offset, int rank, co
                  float q_scale, float* out, int entries, int heads, int dim, int vdim, int tokens, float* runs,
                  float* run_decay, hipStream_t stream);
 
+// Several residual streams, per-head norms before the cache, a matrix memory with exponential gates
+// (stream_mixers.hip; the kernels' comments say what each computes).
+int mlr_streams_fill(const float* x, float* out, int tokens, int width, int streams, hipStream_t stream);
+int mlr_streams_step(float* x, int streams, int tokens, int width, const int* rows, int out_rows, const void* y,
+                     int y_is_f32, int slices, const float* mix, const float* out_w, const float* in_w,
+                     const void* norm_w, int norm_is_f32, float eps, void* h_out, float* sum_out, int dtype,
+                     hipStream_t stream);
+int mlr_head_norm_rope_write(const float* projected, int width, void* q_out, float* gate, const float* cos,
+                             const float* sin, int rotary_dims, float eps, const int* slots, void* key_pages,
+                             void* value_pages, float* v_keep, const float* v_first, const float* lambda, int dtype,
+                             int tokens, int heads, int kv_heads, int dim, int vdim, int kernel_dim, int block_size,
+                             int num_pages, hipStream_t stream);
+int mlr_matrix_memory_scan(const float* projected, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
+                           float* state, int state_rows, const int* read_rows, const int* write_rows, const int* cu_q,
+                           const int* q_starts, float cap, float q_scale, float* out, int entries, int heads, int dim,
+                           int vdim, hipStream_t stream);
+
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds
 // uniform[k] * total.  temperature and uniform may be null (all greedy).  `scratch`
@@ -290,7 +307,10 @@ int mlr_sample_static(const float* logits, const float* temperature, const float
 // c; eligible are the experts of the `keep` highest blocks; ids [tokens, top] = arg-top-`top` of c over
 // the eligible (ties to the lower index), weights [tokens, top] = s[id] * scale.
 int mlr_moe_route(const float* logits, const float* correction, int* ids, float* weights, int tokens, int experts,
-                  int top, int groups, int keep, float scale, hipStream_t stream);
+                  int top, int groups, int keep, float scale, int score_kind, int normalise, hipStream_t stream);
+// out[j, t, :] = weights[t, j] * h[t, :] where ids[t, j] >= first: experts without matrices that hand their input on.
+int mlr_moe_identity(const void* h, const int* ids, const float* weights, float* out, int dtype, int tokens, int top,
+                     int hidden, int first, hipStream_t stream);
 // The (token, choice) pairs p = token * top + choice sorted by expert: sorted [pairs], offsets
 // [experts + 1], tiles [max_tiles, 2] = (expert, first row of `sorted`) with up to
 // mlr_moe_tile_rows(big) rows each (16, or 64 with `big`), unused tiles (-1, 0).  max_tiles >=

@@ -23,7 +23,8 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     const int* __restrict__ token_entry, const int* __restrict__ positions, T* __restrict__ out, int entries,
     int heads, int kv_heads, int head_dim, int block_size, int num_pages, float scale, int window, int chunk,
     const float* __restrict__ sinks, const T* __restrict__ pooled_keys, const T* __restrict__ pooled_values,
-    const int* __restrict__ pooled_table, int pooled_width, int pooled_pages, int pool) {
+    const int* __restrict__ pooled_table, int pooled_width, int pooled_pages, int pool,
+    const float* __restrict__ score_bias) {
   __shared__ float qs[MAXD];
   __shared__ float ps[kWave];
   __shared__ int64_t offs[kWave];
@@ -46,6 +47,10 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
   __syncthreads();
 
   const int first = first_visible_key(p, window, chunk);
+  // score_bias: no softmax at all.  A visible key weighs sigmoid(score + score_bias[head]) whatever the other
+  // keys are, and nothing is normalised.
+  const bool gated_keys = score_bias != nullptr;
+  const float bias = gated_keys ? score_bias[h] : 0.f;
   float m = -INFINITY;
   float l = 0.f;
   float acc[MAXD / kWave];
@@ -86,11 +91,17 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
           s = dot;
         }
       }
-      const float m_new = fmaxf(m, wave_max(s));
-      const float pr = (off >= 0) ? expf(s - m_new) : 0.f;
-      const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
-      l = l * alpha + wave_sum(pr);
-      m = m_new;
+      float pr, alpha;
+      if (gated_keys) {
+        pr = (off >= 0) ? 1.0f / (1.0f + expf(-(s + bias))) : 0.f;
+        alpha = 1.0f;
+      } else {
+        const float m_new = fmaxf(m, wave_max(s));
+        pr = (off >= 0) ? expf(s - m_new) : 0.f;
+        alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        l = l * alpha + wave_sum(pr);
+        m = m_new;
+      }
       ps[lane] = pr;
       offs[lane] = off;
       voffs[lane] = voff;
@@ -122,7 +133,7 @@ __global__ __launch_bounds__(64) void paged_attention_simple_kernel(
     for (int j = 0; j < MAXD / kWave; ++j) acc[j] *= alpha;
   }
   const bool any_bad = __any(bad);
-  const float inv = 1.0f / l;
+  const float inv = gated_keys ? 1.0f : 1.0f / l;
 #pragma unroll
   for (int j = 0; j < MAXD / kWave; ++j) {
     const int dim = lane + j * kWave;
@@ -141,7 +152,7 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
                                           int block_size, int num_pages, float scale, int window, int chunk,
                                           const float* sinks, const void* pooled_keys, const void* pooled_values,
                                           const int* pooled_table, int pooled_width, int pooled_pages, int pool,
-                                          hipStream_t stream) {
+                                          const float* score_bias, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && token_entry && positions && out, "null pointer");
   MLR_REQUIRE(tokens > 0 && entries > 0 && heads > 0 && kv_heads > 0, "sizes must be > 0");
   MLR_REQUIRE(heads % kv_heads == 0, "query heads must be a multiple of KV heads");
@@ -155,13 +166,14 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
                                           pooled_pages > 0)),
               "pooled entries need a window, their pages and their table");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  MLR_REQUIRE(score_bias == nullptr || (sinks == nullptr && pool == 0), "keys weighed one by one have no sink and no pooled entries");
   dim3 grid(tokens, heads);
 #define MLR_SIMPLE(T, MAXD)                                                                                      \
   paged_attention_simple_kernel<T, MAXD><<<grid, kWave, 0, stream>>>(                                            \
       static_cast<const T*>(q), q_stride, static_cast<const T*>(key_pages), static_cast<const T*>(value_pages),   \
       block_table, table_width, token_entry, positions, static_cast<T*>(out), entries, heads, kv_heads, head_dim, \
       block_size, num_pages, scale, window, chunk, sinks, static_cast<const T*>(pooled_keys),                    \
-      static_cast<const T*>(pooled_values), pooled_table, pooled_width, pooled_pages, pool)
+      static_cast<const T*>(pooled_values), pooled_table, pooled_width, pooled_pages, pool, score_bias)
   if (head_dim > 256) {
     if (dtype == kF32)
       MLR_SIMPLE(float, kMaxHeadDim);
@@ -176,14 +188,14 @@ extern "C" int mlr_paged_attention_simple(const void* q, int64_t q_stride, const
         static_cast<const float*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<float*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
         sinks, static_cast<const float*>(pooled_keys), static_cast<const float*>(pooled_values), pooled_table,
-        pooled_width, pooled_pages, pool);
+        pooled_width, pooled_pages, pool, score_bias);
   else
     paged_attention_simple_kernel<bf16, 256><<<grid, kWave, 0, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),
         static_cast<const bf16*>(value_pages), block_table, table_width, token_entry, positions,
         static_cast<bf16*>(out), entries, heads, kv_heads, head_dim, block_size, num_pages, scale, window, chunk,
         sinks, static_cast<const bf16*>(pooled_keys), static_cast<const bf16*>(pooled_values), pooled_table,
-        pooled_width, pooled_pages, pool);
+        pooled_width, pooled_pages, pool, score_bias);
   MLR_LAUNCH_CHECK();
   return 0;
 }

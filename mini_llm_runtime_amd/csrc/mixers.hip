@@ -208,10 +208,13 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     float* __restrict__ gate, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims,
     const void* __restrict__ norm_weight, int weight_is_f32, float eps, const int* __restrict__ slots,
     T* __restrict__ key_pages, T* __restrict__ value_pages, int heads, int dim, int rot, int rank, int D,
-    int block_size, int num_pages, int own_cache, int gated) {
+    int block_size, int num_pages, int own_cache, int gated, const float* __restrict__ queries, int q_width) {
   __shared__ float scratch[16];
   const int64_t t = blockIdx.x;
   const float* row = p + t * width;
+  // the query sums: the leading columns of the row, or (a mixer whose queries go through a product of their
+  // own) a row of another tensor, the row then starts with what follows the queries
+  const float* qrow = queries != nullptr ? queries + t * q_width : row;
   const int half = rdims / 2;
   const float* cs = cos_t ? cos_t + t * half : nullptr;
   const float* sn = sin_t ? sin_t + t * half : nullptr;
@@ -222,15 +225,15 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
   const int qd = dim + rot;
   for (int i = threadIdx.x; i < heads * dim; i += 256) {
     const int h = i / dim;
-    q_plain[t * heads * dim + i] = from_f32<T>(row[h * qd + (i - h * dim)]);
+    q_plain[t * heads * dim + i] = from_f32<T>(qrow[h * qd + (i - h * dim)]);
   }
   const int tail = D - rank;  // columns of a latent query that this kernel owns
   for (int i = threadIdx.x; i < heads * tail; i += 256) {
     const int h = i / tail;
     const int j = i - h * tail;
-    q_latent[(t * heads + h) * D + rank + j] = from_f32<T>(j < rot ? rotated(row + h * qd + dim, j) : 0.f);
+    q_latent[(t * heads + h) * D + rank + j] = from_f32<T>(j < rot ? rotated(qrow + h * qd + dim, j) : 0.f);
   }
-  int at = heads * qd;
+  int at = queries != nullptr ? 0 : heads * qd;
   if (own_cache) {
     const float* c = row + at;
     float ss = 0.f;
@@ -754,18 +757,20 @@ __global__ __launch_bounds__(256) void retention_apply_kernel(const float* __res
   }
 }
 
-// out[t, h, :] = o / sqrt(mean(o^2) + eps) * w * silu(z) * out_scale, o = retained[t, h, :] (float32), z = the gate
-// sums at column gate_offset + h * vdim of p [tokens, width] (float32), w [vdim] a weight that all heads share
-// (null: none).  A row of `out` is out_row elements long and the heads start at its column 0.  One wavefront
+// out[t, h, :] = o / sqrt(mean(o^2) + eps) * w * act(z) * out_scale, o = retained[t, h, :] (float32), z = the gate
+// sums at column gate_offset + h * vdim of p [tokens, width] (float32), w [vdim] a weight that all heads share, or
+// with `weight_per_head` [heads * vdim] (null: none); act is silu (gate_kind 0) or the sigmoid (1).  A row of `out` is out_row elements long and the heads start at its column 0.  One wavefront
 // per (token, head).
 template <typename T>
 __global__ __launch_bounds__(64) void retention_gate_kernel(const float* __restrict__ retained,
                                                             const float* __restrict__ p, int width, int gate_offset,
                                                             T* __restrict__ out, int64_t out_row, int heads, int vdim,
                                                             float eps, const void* __restrict__ norm_weight,
-                                                            int weight_is_f32, float out_scale) {
+                                                            int weight_is_f32, float out_scale,
+                                                            int weight_per_head, int gate_kind) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
+  const int w0 = weight_per_head ? h * vdim : 0;
   const float* o = retained + (t * heads + h) * vdim;
   float ss = 0.f;
   for (int i = threadIdx.x; i < vdim; i += 64) ss += o[i] * o[i];
@@ -775,8 +780,9 @@ __global__ __launch_bounds__(64) void retention_gate_kernel(const float* __restr
   for (int i = threadIdx.x; i < vdim; i += 64) {
     const float zv = z[i];
     float normed = o[i] * inv;
-    if (norm_weight != nullptr) normed *= load_as_f32(norm_weight, i, weight_is_f32);
-    dst[i] = from_f32<T>(normed * (zv / (1.0f + expf(-zv))) * out_scale);
+    if (norm_weight != nullptr) normed *= load_as_f32(norm_weight, w0 + i, weight_is_f32);
+    const float sg = 1.0f / (1.0f + expf(-zv));
+    dst[i] = from_f32<T>(normed * (gate_kind ? sg : zv * sg) * out_scale);
   }
 }
 
@@ -832,13 +838,15 @@ int mlr_latent_prepare(const float* projected, int width, void* q_plain, void* q
                        const float* sin, int rotary_dims, const void* norm_weight, int weight_is_f32, float eps,
                        const int* slots, void* key_pages, void* value_pages, int dtype, int tokens, int heads, int dim,
                        int rot, int rank, int kernel_dim, int block_size, int num_pages, int own_cache, int gated,
-                       hipStream_t stream) {
+                       const float* queries, int q_width, hipStream_t stream) {
   MLR_REQUIRE(projected && q_plain && q_latent, "null pointer");
+  MLR_REQUIRE(queries == nullptr || q_width >= heads * (dim + rot), "the query rows are too narrow");
   MLR_REQUIRE(tokens > 0 && heads > 0 && dim > 0 && rot > 0 && rank > 0, "sizes must be > 0");
   MLR_REQUIRE(kernel_dim >= rank + rot, "the kernels' head size must hold latent and rotated part");
   MLR_REQUIRE(rotary_dims >= 0 && rotary_dims % 2 == 0 && rotary_dims <= rot, "rotary_dims must be even and within rot");
   MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
-  MLR_REQUIRE(width >= heads * (dim + rot) + (own_cache ? rank + rot : 0) + (gated ? heads : 0), "the projected rows are too narrow");
+  MLR_REQUIRE(width >= (queries ? 0 : heads * (dim + rot)) + (own_cache ? rank + rot : 0) + (gated ? heads : 0),
+              "the projected rows are too narrow");
   MLR_REQUIRE(!own_cache || (norm_weight && slots && key_pages && value_pages && block_size > 0 && num_pages > 0),
               "a cache write needs the latent's norm weight, slots, pages and their sizes");
   MLR_REQUIRE(!gated || gate, "a gated mixer needs room for its gates");
@@ -847,12 +855,12 @@ int mlr_latent_prepare(const float* projected, int width, void* q_plain, void* q
     latent_prepare_kernel<float><<<tokens, 256, 0, stream>>>(
         projected, width, static_cast<float*>(q_plain), static_cast<float*>(q_latent), gate, cos, sin, rotary_dims,
         norm_weight, weight_is_f32, eps, slots, static_cast<float*>(key_pages), static_cast<float*>(value_pages), heads,
-        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated);
+        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated, queries, q_width);
   else
     latent_prepare_kernel<bf16><<<tokens, 256, 0, stream>>>(
         projected, width, static_cast<bf16*>(q_plain), static_cast<bf16*>(q_latent), gate, cos, sin, rotary_dims,
         norm_weight, weight_is_f32, eps, slots, static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages), heads,
-        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated);
+        dim, rot, rank, kernel_dim, block_size, num_pages, own_cache, gated, queries, q_width);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -975,8 +983,9 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
 
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
                        int tokens, int heads, int vdim, float eps, const void* norm_weight, int weight_is_f32,
-                       float out_scale, int64_t out_row, hipStream_t stream) {
+                       float out_scale, int64_t out_row, int weight_per_head, int gate_kind, hipStream_t stream) {
   MLR_REQUIRE(retained && projected && out, "null pointer");
+  MLR_REQUIRE(gate_kind == 0 || gate_kind == 1, "the gate is silu (0) or the sigmoid (1)");
   MLR_REQUIRE(tokens > 0 && heads > 0 && heads < 65536 && vdim > 0, "sizes must be > 0");
   MLR_REQUIRE(gate_offset >= 0 && width >= gate_offset + heads * vdim, "the projected rows do not hold the gate");
   MLR_REQUIRE(out_row >= static_cast<int64_t>(heads) * vdim, "a row of the output is shorter than the heads");
@@ -985,11 +994,12 @@ int mlr_retention_gate(const float* retained, const float* projected, int width,
   if (dtype == kF32)
     retention_gate_kernel<float><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
                                                           static_cast<float*>(out), out_row, heads, vdim, eps,
-                                                          norm_weight, weight_is_f32, out_scale);
+                                                          norm_weight, weight_is_f32, out_scale, weight_per_head, gate_kind);
   else
     retention_gate_kernel<bf16><<<grid, 64, 0, stream>>>(retained, projected, width, gate_offset,
                                                          static_cast<bf16*>(out), out_row, heads, vdim, eps,
-                                                         norm_weight, weight_is_f32, out_scale);
+                                                         norm_weight, weight_is_f32, out_scale, weight_per_head,
+                                                         gate_kind);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -29,14 +29,16 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// One wavefront per token.  s = sigmoid(z), c = s + correction; block g of experts / groups
+// One wavefront per token.  s = sigmoid(z) (score_kind 0) or softmax(z) over all experts (1), c = s + correction;
+// with `normalise` the chosen weights are divided by their sum (+ 1e-20) before the scale.  Block g of experts / groups
 // consecutive experts scores top-2 sum of its c; c := -inf outside the `keep` highest blocks; then
 // `top` rounds of arg-max over c (ties to the lower index), each winner e leaving ids = e and
 // weights = s[e] * scale.
 __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restrict__ logits,
                                                           const float* __restrict__ correction,
                                                           int* __restrict__ ids, float* __restrict__ weights,
-                                                          int experts, int top, int groups, int keep, float scale) {
+                                                          int experts, int top, int groups, int keep, float scale,
+                                                          int score_kind, int normalise) {
   extern __shared__ float route_lds[];
   float* c = route_lds;            // [experts]
   float* s = route_lds + experts;  // [experts]
@@ -45,8 +47,17 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
   const int lane = threadIdx.x;
   const int per = experts / groups;
   const float* z = logits + static_cast<int64_t>(t) * experts;
+  float z_max = 0.f, z_inv = 1.f;
+  if (score_kind == 1) {
+    float mx = -INFINITY;
+    for (int e = lane; e < experts; e += kWave) mx = fmaxf(mx, z[e]);
+    z_max = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < experts; e += kWave) sum += expf(z[e] - z_max);
+    z_inv = 1.0f / wave_sum(sum);
+  }
   for (int e = lane; e < experts; e += kWave) {
-    const float sv = 1.0f / (1.0f + expf(-z[e]));
+    const float sv = score_kind == 1 ? expf(z[e] - z_max) * z_inv : 1.0f / (1.0f + expf(-z[e]));
     s[e] = sv;
     c[e] = sv + (correction != nullptr ? correction[e] : 0.f);
   }
@@ -85,6 +96,7 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
       if (gs[e / per] != INFINITY) c[e] = -INFINITY;
     __syncthreads();
   }
+  float chosen_sum = 0.f;
   for (int k = 0; k < top; ++k) {
     float v = -INFINITY;
     int i = 0x7fffffff;
@@ -97,6 +109,7 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
     }
     wave_argmax(v, i);
     if (i >= experts) i = 0;  // only if every score left is NaN or -inf: keep the id in range
+    chosen_sum += s[i];
     if (lane == 0) {
       ids[static_cast<int64_t>(t) * top + k] = i;
       weights[static_cast<int64_t>(t) * top + k] = s[i] * scale;
@@ -104,6 +117,26 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
     }
     __syncthreads();
   }
+  if (normalise) {
+    const float inv = 1.0f / (chosen_sum + 1e-20f);
+    for (int k = lane; k < top; k += kWave) weights[static_cast<int64_t>(t) * top + k] *= inv;
+  }
+}
+
+// Experts that hand their input on: where ids[t, j] >= first (such an expert has no matrices and the grouped
+// products skip its pairs) out[j, t, :] = weights[t, j] * h[t, :].  One workgroup per pair.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_identity_kernel(const T* __restrict__ h, const int* __restrict__ ids,
+                                                           const float* __restrict__ weights, float* __restrict__ out,
+                                                           int tokens, int top, int hidden, int first) {
+  const int pair = blockIdx.x;
+  if (ids[pair] < first) return;
+  const int t = pair / top;
+  const int j = pair - t * top;
+  const float w = weights[pair];
+  const T* src = h + static_cast<int64_t>(t) * hidden;
+  float* dst = out + (static_cast<int64_t>(j) * tokens + t) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += 256) dst[i] = w * to_f32(src[i]);
 }
 
 // ---- pairs sorted by expert ------------------------------------------------------------------
@@ -617,14 +650,31 @@ using namespace mlr;
 extern "C" {
 
 int mlr_moe_route(const float* logits, const float* correction, int* ids, float* weights, int tokens, int experts,
-                  int top, int groups, int keep, float scale, hipStream_t stream) {
+                  int top, int groups, int keep, float scale, int score_kind, int normalise, hipStream_t stream) {
   MLR_REQUIRE(logits && ids && weights, "null pointer");
+  MLR_REQUIRE(score_kind == 0 || score_kind == 1, "scores are sigmoids (0) or a softmax (1)");
   MLR_REQUIRE(tokens > 0 && experts > 0 && top > 0 && top <= experts, "sizes must be > 0 and top <= experts");
   MLR_REQUIRE(groups > 0 && experts % groups == 0 && keep > 0 && keep <= groups, "bad groups");
   MLR_REQUIRE(top <= keep * (experts / groups), "the kept groups hold fewer experts than a token uses");
   MLR_REQUIRE(experts <= 4096, "at most 4096 experts");
   const size_t lds = (2 * static_cast<size_t>(experts) + groups) * sizeof(float);
-  moe_route_kernel<<<tokens, kWave, lds, stream>>>(logits, correction, ids, weights, experts, top, groups, keep, scale);
+  moe_route_kernel<<<tokens, kWave, lds, stream>>>(logits, correction, ids, weights, experts, top, groups, keep, scale,
+                                                   score_kind, normalise);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_moe_identity(const void* h, const int* ids, const float* weights, float* out, int dtype, int tokens, int top,
+                     int hidden, int first, hipStream_t stream) {
+  MLR_REQUIRE(h && ids && weights && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && top > 0 && hidden > 0 && first >= 0, "sizes must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    moe_identity_kernel<float><<<tokens * top, 256, 0, stream>>>(static_cast<const float*>(h), ids, weights, out, tokens,
+                                                                 top, hidden, first);
+  else
+    moe_identity_kernel<bf16><<<tokens * top, 256, 0, stream>>>(static_cast<const bf16*>(h), ids, weights, out, tokens,
+                                                                top, hidden, first);
   MLR_LAUNCH_CHECK();
   return 0;
 }

@@ -1,0 +1,368 @@
+// Several residual streams side by side (hyper-connections), the preparation of an attention whose
+// queries, keys and values are normed per head, and a matrix memory with exponential gates.
+// Everything here is 32-bit inside; activations leave in the engine's dtype.
+#include "api.h"
+#include "common.h"
+
+namespace mlr {
+
+constexpr int kMaxStreams = 16;
+
+// ---- residual streams -------------------------------------------------------------------------------
+// x [streams, tokens, width] float32.  One workgroup per output row r (token rows[r], or r).  In order:
+//  1. (y given) all streams at once from the old ones: x_t = sum_s mix[s, t] x_s + out_w[t] * y, y a row of
+//     activations (engine dtype or float32) or the sum, in order, of `slices` float32 rows; written back
+//     unless `rows` choose tokens (then the streams stay as they are and only the outputs below are made);
+//  2. u = sum_s in_w[s] x_s (in_w null: the plain sum of the streams);
+//  3. (sum_out) u as float32; (h_out) u * rsqrt(mean(u^2) + eps) * norm_w in the engine's dtype.
+template <typename T>
+__global__ __launch_bounds__(256) void streams_step_kernel(
+    float* __restrict__ x, int streams, int tokens, int width, const int* __restrict__ rows, const void* __restrict__ y,
+    int y_is_f32, int slices, const float* __restrict__ mix, const float* __restrict__ out_w,
+    const float* __restrict__ in_w, const void* __restrict__ norm_w, int norm_is_f32, float eps, T* __restrict__ h_out,
+    float* __restrict__ sum_out) {
+  __shared__ float scratch[16];
+  __shared__ float s_mix[kMaxStreams * kMaxStreams];
+  __shared__ float s_out[kMaxStreams];
+  __shared__ float s_in[kMaxStreams];
+  const int r = blockIdx.x;
+  const int64_t t = rows != nullptr ? rows[r] : r;
+  const bool write_back = rows == nullptr;
+  const int64_t plane = static_cast<int64_t>(tokens) * width;
+  for (int i = threadIdx.x; i < streams * streams; i += 256) s_mix[i] = mix != nullptr ? mix[i] : 0.f;
+  for (int i = threadIdx.x; i < streams; i += 256) {
+    s_out[i] = out_w != nullptr ? out_w[i] : 0.f;
+    s_in[i] = in_w != nullptr ? in_w[i] : 1.f;
+  }
+  __syncthreads();
+  float ss = 0.f;
+  for (int pass = 0; pass < 2; ++pass) {
+    // the second pass makes the same numbers again (from the old streams when nothing was written back)
+    if (pass == 1 && h_out == nullptr) break;
+    float inv = 0.f;
+    if (pass == 1) inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps);
+    for (int c = threadIdx.x; c < width; c += 256) {
+      float xs[kMaxStreams];
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s) xs[s] = s < streams ? x[s * plane + t * width + c] : 0.f;
+      float u = 0.f;
+      if (y != nullptr && !(pass == 1 && write_back)) {
+        float yv = 0.f;
+        if (slices > 0) {
+          for (int k = 0; k < slices; ++k) yv += static_cast<const float*>(y)[k * plane + t * width + c];
+        } else {
+          yv = load_as_f32(y, t * width + c, y_is_f32);
+        }
+#pragma unroll
+        for (int to = 0; to < kMaxStreams; ++to) {
+          if (to < streams) {
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < kMaxStreams; ++s)
+              if (s < streams) v = fmaf(s_mix[s * streams + to], xs[s], v);
+            v = fmaf(s_out[to], yv, v);
+            if (write_back) x[to * plane + t * width + c] = v;
+            u = fmaf(s_in[to], v, u);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < kMaxStreams; ++s)
+          if (s < streams) u = fmaf(s_in[s], xs[s], u);
+      }
+      if (pass == 0) {
+        ss += u * u;
+        if (sum_out != nullptr) sum_out[static_cast<int64_t>(r) * width + c] = u;
+      } else {
+        h_out[static_cast<int64_t>(r) * width + c] = from_f32<T>(u * inv * load_as_f32(norm_w, c, norm_is_f32));
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void streams_fill_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                           int64_t plane, int streams) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= plane) return;
+  const float v = x[i];
+  for (int s = 0; s < streams; ++s) out[s * plane + i] = v;
+}
+
+// ---- queries, keys and values normed per head -----------------------------------------------------------
+// p [tokens, width] float32 holds per token: heads * dim query sums, kv_heads * dim key sums, kv_heads * vdim value
+// sums, then `heads` gate logits (if gate is given).  Per token:
+//  * every query and key head: rotation of its first rdims dims in two halves (pair j, j + rdims / 2), then the
+//    head divided by its root mean square over dim (eps inside the root); queries to q_out [tokens, heads * D]
+//    (columns dim .. D - 1 zero), keys to the key pages [page, kv_head, offset, D] at slot[t];
+//  * every value head divided by its root mean square over vdim; (v_keep) the normed values as float32 [tokens,
+//    kv_heads * vdim]; (v_first) v = (1 - lambda) v + lambda v_first[t]; values to [page, kv_head, D, offset];
+//  * gate[t, head] = sigmoid(logit).
+// One wavefront per head; a negative slot stores nothing.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_rope_write_kernel(
+    const float* __restrict__ p, int width, T* __restrict__ q_out, float* __restrict__ gate,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rdims, float eps,
+    const int* __restrict__ slots, T* __restrict__ key_pages, T* __restrict__ value_pages, float* __restrict__ v_keep,
+    const float* __restrict__ v_first, const float* __restrict__ lambda_p, int heads, int kv_heads, int dim, int vdim,
+    int D, int block_size, int num_pages) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const float* row = p + t * width;
+  const int half = rdims / 2;
+  const float* cs = cos_t != nullptr ? cos_t + t * half : nullptr;
+  const float* sn = sin_t != nullptr ? sin_t + t * half : nullptr;
+  const int slot = slots[t];
+  const int page = slot >= 0 ? slot / block_size : -1;
+  const int off = slot >= 0 ? slot - page * block_size : 0;
+  const bool store = page >= 0 && page < num_pages;
+  const float lambda = (v_first != nullptr && lambda_p != nullptr) ? lambda_p[0] : 0.f;
+  const int jobs = heads + 2 * kv_heads;
+  for (int job = wave; job < jobs; job += 4) {
+    const bool is_q = job < heads;
+    const bool is_k = !is_q && job < heads + kv_heads;
+    const int h = is_q ? job : (is_k ? job - heads : job - heads - kv_heads);
+    const int n = (is_q || is_k) ? dim : vdim;
+    const float* src = row + (is_q ? h * dim : (is_k ? heads * dim + h * dim : (heads + kv_heads) * dim + h * vdim));
+    auto value = [&](int j) {
+      if (!(is_q || is_k) || j >= rdims || cs == nullptr) return src[j];
+      return j < half ? src[j] * cs[j] - src[j + half] * sn[j] : src[j] * cs[j - half] + src[j - half] * sn[j - half];
+    };
+    float ss = 0.f;
+    for (int j = lane; j < n; j += kWave) {
+      const float v = value(j);
+      ss += v * v;
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(n) + eps);
+    if (is_q) {
+      T* dst = q_out + (t * heads + h) * D;
+      for (int j = lane; j < D; j += kWave) dst[j] = from_f32<T>(j < n ? value(j) * inv : 0.f);
+    } else if (is_k) {
+      if (store) {
+        T* dst = key_pages + ((static_cast<int64_t>(page) * kv_heads + h) * block_size + off) * D;
+        for (int j = lane; j < D; j += kWave) dst[j] = from_f32<T>(j < n ? value(j) * inv : 0.f);
+      }
+    } else {
+      T* dst = value_pages + (static_cast<int64_t>(page) * kv_heads + h) * D * block_size + off;
+      for (int j = lane; j < D; j += kWave) {
+        float v = 0.f;
+        if (j < n) {
+          v = src[j] * inv;
+          if (v_keep != nullptr) v_keep[(t * kv_heads + h) * vdim + j] = v;
+          if (v_first != nullptr) v = (1.0f - lambda) * v + lambda * v_first[(t * kv_heads + h) * vdim + j];
+        }
+        if (store) dst[static_cast<int64_t>(j) * block_size] = from_f32<T>(v);
+      }
+    }
+  }
+  if (gate != nullptr) {
+    const float* z = row + (heads + kv_heads) * dim + kv_heads * vdim;
+    for (int h = threadIdx.x; h < heads; h += 256) gate[t * heads + h] = 1.0f / (1.0f + expf(-z[h]));
+  }
+}
+
+// ---- matrix memory with exponential gates ------------------------------------------------------------------
+// Per head: a matrix C [dim, vdim], a vector n [dim] and a running maximum m, all float32, in `state` [state_rows,
+// heads, dim * vdim + dim + 1] (C row-major, then n, then m).  Per token, with a = the input gate's sum and b = the
+// forget gate's sum (both with their biases):
+//   i = cap tanh(a / cap),  f = logsigmoid(cap tanh(b / cap)),  m' = max(f + m, i),
+//   C' = exp(f + m - m') C + exp(i - m') k v^T,  n' likewise with k alone,
+//   o = C'^T q / (max(|n' . q|, exp(-m')) + 1e-6),  q scaled by q_scale.
+// An entry that starts its request starts from zeros (m = 0 too) whatever its row holds.  A workgroup of four
+// wavefronts owns 64 value columns of one head of one entry: lane (g, c) of a wavefront holds rows g, g + 4, ... of
+// column c of C and the same rows of n; eight tokens' q and k at a time go through LDS, rows beyond dim as zeros,
+// so the inner loops have no conditions.
+constexpr int kMemTokens = 8;
+
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <int R>  // rows of the state a lane holds: dim <= 4 * R
+__global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
+    const float* __restrict__ p, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
+    float* __restrict__ state, const int* __restrict__ read_rows, const int* __restrict__ write_rows,
+    const int* __restrict__ cu_q, const int* __restrict__ q_starts, float cap, float q_scale, float* __restrict__ out,
+    int heads, int dim, int vdim) {
+  constexpr int MAXD = 4 * R;
+  __shared__ __attribute__((aligned(16))) float sq[kMemTokens][MAXD];
+  __shared__ __attribute__((aligned(16))) float sk[kMemTokens][MAXD];
+  __shared__ float sv[kMemTokens][64];
+  __shared__ float sg[kMemTokens][2];
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int g = lane / 16;
+  const int c_local = wave * 16 + lane % 16;
+  const int col = blockIdx.z * 64 + c_local;
+  const bool col_ok = col < vdim;
+  const int t_begin = cu_q[entry];
+  const int t_end = cu_q[entry + 1];
+  const int64_t per_head = static_cast<int64_t>(dim) * vdim + dim + 1;
+  const bool fresh = q_starts[entry] == 0;
+  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * per_head;
+  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * per_head;
+
+  float C[R], n[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int r = g + 4 * j;
+    const bool in = r < dim && !fresh;
+    C[j] = (in && col_ok) ? src[static_cast<int64_t>(r) * vdim + col] : 0.f;
+    n[j] = in ? src[static_cast<int64_t>(dim) * vdim + r] : 0.f;
+  }
+  float m = fresh ? 0.f : src[static_cast<int64_t>(dim) * vdim + dim];
+
+  for (int t0 = t_begin; t0 < t_end; t0 += kMemTokens) {
+    const int nb = min(kMemTokens, t_end - t0);
+    __syncthreads();
+    for (int idx = tid; idx < nb * MAXD; idx += 256) {
+      const int tt = idx / MAXD;
+      const int r = idx - tt * MAXD;
+      const float* row = p + static_cast<int64_t>(t0 + tt) * width;
+      sq[tt][r] = r < dim ? row[q_off + h * dim + r] * q_scale : 0.f;
+      sk[tt][r] = r < dim ? row[k_off + h * dim + r] : 0.f;
+    }
+    for (int idx = tid; idx < nb * 64; idx += 256) {
+      const int tt = idx / 64;
+      const int c = blockIdx.z * 64 + (idx - tt * 64);
+      sv[tt][idx - tt * 64] = c < vdim ? p[static_cast<int64_t>(t0 + tt) * width + v_off + h * vdim + c] : 0.f;
+    }
+    if (tid < nb) {
+      const float* row = p + static_cast<int64_t>(t0 + tid) * width;
+      sg[tid][0] = cap * tanhf(row[i_off + h] / cap);
+      sg[tid][1] = log_sigmoid(cap * tanhf(row[f_off + h] / cap));
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nb; ++tt) {
+      const float ig = sg[tt][0];
+      const float fg = sg[tt][1];
+      const float m_new = fmaxf(fg + m, ig);
+      const float keep = expf(fg + m - m_new);
+      const float take = expf(ig - m_new);
+      m = m_new;
+      const float v = sv[tt][c_local] * take;
+      float num = 0.f, nq = 0.f;
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const float kv = sk[tt][g + 4 * j];
+        const float qv = sq[tt][g + 4 * j];
+        C[j] = fmaf(keep, C[j], kv * v);
+        n[j] = fmaf(keep, n[j], kv * take);
+        num = fmaf(C[j], qv, num);
+        nq = fmaf(n[j], qv, nq);
+      }
+      num += __shfl_xor(num, 16, kWave);
+      num += __shfl_xor(num, 32, kWave);
+      nq += __shfl_xor(nq, 16, kWave);
+      nq += __shfl_xor(nq, 32, kWave);
+      if (g == 0 && col_ok)
+        out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int r = g + 4 * j;
+    if (r < dim) {
+      if (col_ok) dst[static_cast<int64_t>(r) * vdim + col] = C[j];
+      if (blockIdx.z == 0 && wave == 0 && lane % 16 == 0) dst[static_cast<int64_t>(dim) * vdim + r] = n[j];
+    }
+  }
+  if (blockIdx.z == 0 && tid == 0) dst[static_cast<int64_t>(dim) * vdim + dim] = m;
+}
+
+}  // namespace mlr
+
+using namespace mlr;
+
+extern "C" {
+
+int mlr_streams_fill(const float* x, float* out, int tokens, int width, int streams, hipStream_t stream) {
+  MLR_REQUIRE(x && out, "null pointer");
+  MLR_REQUIRE(tokens > 0 && width > 0 && streams > 0 && streams <= kMaxStreams, "sizes must be > 0, at most 16 streams");
+  const int64_t plane = static_cast<int64_t>(tokens) * width;
+  streams_fill_kernel<<<static_cast<unsigned>((plane + 255) / 256), 256, 0, stream>>>(x, out, plane, streams);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_streams_step(float* x, int streams, int tokens, int width, const int* rows, int out_rows, const void* y,
+                     int y_is_f32, int slices, const float* mix, const float* out_w, const float* in_w,
+                     const void* norm_w, int norm_is_f32, float eps, void* h_out, float* sum_out, int dtype,
+                     hipStream_t stream) {
+  MLR_REQUIRE(x, "null pointer");
+  MLR_REQUIRE(tokens > 0 && width > 0 && streams > 0 && streams <= kMaxStreams, "sizes must be > 0, at most 16 streams");
+  MLR_REQUIRE(out_rows > 0 && (rows != nullptr || out_rows == tokens), "without chosen rows every token is a row");
+  MLR_REQUIRE(y == nullptr || (mix && out_w), "an update needs its mixing matrix and output weights");
+  MLR_REQUIRE(slices >= 0 && (slices == 0 || (y && y_is_f32)), "partial sums are float32");
+  MLR_REQUIRE(h_out == nullptr || norm_w, "normed activations need a norm weight");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    streams_step_kernel<float><<<out_rows, 256, 0, stream>>>(x, streams, tokens, width, rows, y, y_is_f32, slices, mix,
+                                                             out_w, in_w, norm_w, norm_is_f32, eps,
+                                                             static_cast<float*>(h_out), sum_out);
+  else
+    streams_step_kernel<bf16><<<out_rows, 256, 0, stream>>>(x, streams, tokens, width, rows, y, y_is_f32, slices, mix,
+                                                            out_w, in_w, norm_w, norm_is_f32, eps,
+                                                            static_cast<bf16*>(h_out), sum_out);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_head_norm_rope_write(const float* projected, int width, void* q_out, float* gate, const float* cos,
+                             const float* sin, int rotary_dims, float eps, const int* slots, void* key_pages,
+                             void* value_pages, float* v_keep, const float* v_first, const float* lambda, int dtype,
+                             int tokens, int heads, int kv_heads, int dim, int vdim, int kernel_dim, int block_size,
+                             int num_pages, hipStream_t stream) {
+  MLR_REQUIRE(projected && q_out && slots && key_pages && value_pages, "null pointer");
+  MLR_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0, "sizes must be > 0");
+  MLR_REQUIRE(kernel_dim >= dim && kernel_dim >= vdim, "the kernels' head size must hold keys and values");
+  MLR_REQUIRE(rotary_dims >= 0 && rotary_dims % 2 == 0 && rotary_dims <= dim, "rotary_dims must be even and within dim");
+  MLR_REQUIRE(rotary_dims == 0 || (cos && sin), "a rotation needs cos and sin tables");
+  MLR_REQUIRE(width >= (heads + kv_heads) * dim + kv_heads * vdim + (gate ? heads : 0), "the projected rows are too narrow");
+  MLR_REQUIRE(v_first == nullptr || lambda, "mixing values in needs its weight");
+  MLR_REQUIRE(block_size > 0 && num_pages > 0, "page sizes must be > 0");
+  MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (dtype == kF32)
+    head_norm_rope_write_kernel<float><<<tokens, 256, 0, stream>>>(
+        projected, width, static_cast<float*>(q_out), gate, cos, sin, rotary_dims, eps, slots,
+        static_cast<float*>(key_pages), static_cast<float*>(value_pages), v_keep, v_first, lambda, heads, kv_heads, dim,
+        vdim, kernel_dim, block_size, num_pages);
+  else
+    head_norm_rope_write_kernel<bf16><<<tokens, 256, 0, stream>>>(
+        projected, width, static_cast<bf16*>(q_out), gate, cos, sin, rotary_dims, eps, slots,
+        static_cast<bf16*>(key_pages), static_cast<bf16*>(value_pages), v_keep, v_first, lambda, heads, kv_heads, dim,
+        vdim, kernel_dim, block_size, num_pages);
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+int mlr_matrix_memory_scan(const float* projected, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
+                           float* state, int state_rows, const int* read_rows, const int* write_rows, const int* cu_q,
+                           const int* q_starts, float cap, float q_scale, float* out, int entries, int heads, int dim,
+                           int vdim, hipStream_t stream) {
+  MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && out, "null pointer");
+  MLR_REQUIRE(entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
+  MLR_REQUIRE(dim <= 256, "heads of up to 256 dims");
+  MLR_REQUIRE(cap > 0.f, "the gates' cap must be > 0");
+  MLR_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && i_off >= 0 && f_off >= 0 && q_off + heads * dim <= width &&
+                  k_off + heads * dim <= width && v_off + heads * vdim <= width && i_off + heads <= width &&
+                  f_off + heads <= width,
+              "the projected rows do not hold what the offsets name");
+  const dim3 grid(entries, heads, (vdim + 63) / 64);
+#define MLR_MEMORY(R)                                                                                               \
+  matrix_memory_scan_kernel<R><<<grid, 256, 0, stream>>>(projected, width, q_off, k_off, v_off, i_off, f_off, state, \
+                                                         read_rows, write_rows, cu_q, q_starts, cap, q_scale, out,   \
+                                                         heads, dim, vdim)
+  if (dim <= 64)
+    MLR_MEMORY(16);
+  else if (dim <= 128)
+    MLR_MEMORY(32);
+  else
+    MLR_MEMORY(64);
+#undef MLR_MEMORY
+  MLR_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

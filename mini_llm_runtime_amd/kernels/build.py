@@ -67,6 +67,7 @@ CORE = Module(
         "moe.hip",
         "mixers.hip",
         "side_mixers.hip",
+        "stream_mixers.hip",
         "sampling.hip",
     ),
 )

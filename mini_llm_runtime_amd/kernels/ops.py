@@ -32,15 +32,25 @@ _SIGNATURES = {
     "mlr_add_normed": ([_VP, _VP, _I, _I, _VP, _I, _F, _VP, _I, _F, _I, _VP, _I, _I, _I, _VP], _I),
     "mlr_glu_clamped": ([_VP, _I, _VP, _I, _I, _I, _F, _F, _VP], _I),
     "mlr_latent_prepare": (
-        [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
+        [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP,
+         _I, _VP],
         _I,
     ),
+    "mlr_streams_fill": ([_VP, _VP, _I, _I, _I, _VP], _I),
+    "mlr_streams_step": ([_VP, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _F, _VP, _VP, _I, _VP], _I),
+    "mlr_head_norm_rope_write": (
+        [_VP, _I, _VP, _VP, _VP, _VP, _I, _F, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I,
+    ),
+    "mlr_matrix_memory_scan": (
+        [_VP, _I, _I, _I, _I, _I, _I, _VP, _I, _VP, _VP, _VP, _VP, _F, _F, _VP, _I, _I, _I, _I, _VP], _I,
+    ),
+    "mlr_moe_identity": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_retention_scan": (
         [_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _F, _VP, _I, _I, _I, _I, _I, _I, _VP, _I64, _VP], _I,
     ),
     "mlr_retention_scratch": ([_I, _I, _I, _I, _I], _I64),
-    "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP, _I, _F, _I64, _VP], _I),
+    "mlr_retention_gate": ([_VP, _VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP, _I, _F, _I64, _I, _I, _VP], _I),
     "mlr_short_conv": ([_VP, _VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_qk_norm_rope_write": (
         [_VP, _I, _VP, _VP, _I, _F, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP],
@@ -64,7 +74,7 @@ _SIGNATURES = {
     "mlr_qkv_finish": ([_VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_gemm_simple": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _F, _F, _VP], _I),
     "mlr_gemm_bf16": ([_VP, _VP, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _I, _F, _VP, _VP, _F, _F, _VP], _I),
-    "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP], _I),
+    "mlr_moe_route": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _VP], _I),
     "mlr_moe_tile_rows": ([_I], _I),
     "mlr_moe_max_tiles": ([_I, _I, _I], _I),
     "mlr_moe_align": ([_VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP], _I),
@@ -88,7 +98,7 @@ _SIGNATURES = {
     "mlr_gemm_merge_fused_bf16": ([_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I, _VP, _I, _I, _I, _I, _VP], _I),
     "mlr_paged_attention_simple": (
         [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _VP, _VP, _VP, _VP,
-         _I, _I, _I, _VP],
+         _I, _I, _I, _VP, _VP],
         _I,
     ),
     "mlr_sample": ([_VP, _VP, _VP, _VP, _VP, _I, _I, _VP], _I),
@@ -897,8 +907,12 @@ class HipOps:
         chunk: Optional[int] = None,
         sinks: Optional[torch.Tensor] = None,
         pooled: Optional[tuple] = None,
+        score_bias: Optional[torch.Tensor] = None,
     ):
         """Causal attention of the step's tokens over their requests' pages.
+
+        score_bias: float32 [num_heads]; no softmax then: a visible key weighs sigmoid(score * scale +
+        score_bias[head]) whatever the other keys are, and the weights are not normalised.
 
         pooled: (key pages, value pages, block table, pool) of a second set of pages that holds ONE key and
         value for every run of `pool` positions (see `pool_kv_write`); with a window, a query at position p
@@ -945,6 +959,10 @@ class HipOps:
         chunk = int(chunk or 0)
         if sinks is not None:
             self._check(sinks, "sinks", torch.float32, (num_heads,))
+        if score_bias is not None:
+            self._check(score_bias, "score bias", torch.float32, (num_heads,))
+            if sinks is not None or pooled is not None:
+                raise KernelError("keys weighed one by one have no sink and no pooled entries")
         out = self._empty((tokens, num_heads * head_dim), self.dtype)
         width = block_table.shape[1]
         pooled_keys = pooled_values = pooled_table = None
@@ -966,6 +984,7 @@ class HipOps:
             and 16 <= head_dim <= 256
             and block_size % 4 == 0
             and stride % 8 == 0
+            and score_bias is None
         )
         num_tiles = int(getattr(plan, "num_query_tiles", 0))
         num_decode = int(getattr(plan, "num_decode_entries", 0))
@@ -982,7 +1001,8 @@ class HipOps:
                 self._ptr(block_table), width, self._ptr(ctx.token_entry), self._ptr(ctx.positions),
                 self._ptr(out), self.code, tokens, entries, num_heads, num_kv_heads, head_dim, block_size,
                 num_pages, float(scale), int(window or 0), chunk, self._ptr(sinks), self._ptr(pooled_keys),
-                self._ptr(pooled_values), self._ptr(pooled_table), pooled_width, pooled_pages, pool, self._stream(),
+                self._ptr(pooled_values), self._ptr(pooled_table), pooled_width, pooled_pages, pool,
+                self._ptr(score_bias), self._stream(),
             )
             return out
         self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
@@ -1099,15 +1119,20 @@ class HipOps:
         value_pages: torch.Tensor,
         block_size: int,
         kernel_dim: int,
+        queries: Optional[torch.Tensor] = None,
     ):
         """From a latent-attention layer's input sums (float32 [T, heads * (head_dim + rot_dim) (+ kv_rank +
         rot_dim) (+ heads)]: queries, own latent and shared key part, gate logits) to what its kernels take:
         (unrotated query parts [T, heads * head_dim]; latent queries [T, heads * kernel_dim] whose columns
         kv_rank .. kv_rank + rot_dim hold the rotated query parts and whose first kv_rank are left to
         `heads_linear`; gates sigmoid(logit), float32 [T, heads], or None).  With `own_cache` the normed latent
-        and the rotated key part go into the pages: key rows [latent ; key part ; 0], values [latent ; 0]."""
+        and the rotated key part go into the pages: key rows [latent ; key part ; 0], values [latent ; 0].
+        queries: float32 [T, heads * (head_dim + rot_dim)] when the query sums come from a product of their own;
+        `projected` then starts with the latent."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
+        if queries is not None:
+            self._check(queries, "query sums", torch.float32, (tokens, None))
         cos = sin = None
         rotary = 0
         if rotation is not None:
@@ -1128,7 +1153,8 @@ class HipOps:
             int(own_cache and norm_weight.dtype == torch.float32), float(eps),
             self._ptr(slot_mapping if own_cache else None), self._ptr(key_pages if own_cache else None),
             self._ptr(value_pages if own_cache else None), self.code, tokens, heads, head_dim, rot_dim, kv_rank,
-            kernel_dim, block_size, num_pages, int(own_cache), int(gated), self._stream(),
+            kernel_dim, block_size, num_pages, int(own_cache), int(gated), self._ptr(queries),
+            int(queries.shape[1]) if queries is not None else 0, self._stream(),
         )
         return q_plain, q_latent, gate
 
@@ -1236,9 +1262,11 @@ class HipOps:
         scale: float = 1.0,
         out: Optional[torch.Tensor] = None,
         column: int = 0,
+        gate: str = "silu",
     ) -> torch.Tensor:
         """Every head's retained[t, h, :] divided by its root mean square (eps inside the root), times
-        `norm_weight` [value_dim] (one weight for all heads; None: none), times silu of the gate sums in columns
+        `norm_weight` [value_dim] (one weight for all heads) or [heads * value_dim] (None: none), times `gate`
+        ("silu" or "sigmoid") of the gate sums in columns
         gate_offset .. of `projected`, times `scale`; [T, heads * value_dim] in the engine's dtype, or written
         into columns column .. of the wider `out` [T, K]."""
         self._check(projected, "projected input", torch.float32, (None, None))
@@ -1246,13 +1274,17 @@ class HipOps:
         self._check(retained, "retained", torch.float32, (tokens, heads * value_dim))
         if gate_offset < 0 or gate_offset + heads * value_dim > width:
             raise KernelError("the projected rows do not hold the gate")
+        if gate not in ("silu", "sigmoid"):
+            raise KernelError("the gate is 'silu' or 'sigmoid'")
+        per_head = norm_weight is not None and heads > 1 and norm_weight.numel() == heads * value_dim
         if norm_weight is not None:
-            self._check(norm_weight, "head norm weight", (torch.float32, self.dtype), (value_dim,))
+            self._check(norm_weight, "head norm weight", (torch.float32, self.dtype), (heads * value_dim if per_head else value_dim,))
         out, view, row = self._columns(out, column, tokens, heads * value_dim)
         self._call(
             "mlr_retention_gate", self._ptr(retained), self._ptr(projected), width, int(gate_offset), view,
             self.code, tokens, heads, value_dim, float(eps), self._ptr(norm_weight),
-            int(norm_weight is not None and norm_weight.dtype == torch.float32), float(scale), row, self._stream(),
+            int(norm_weight is not None and norm_weight.dtype == torch.float32), float(scale), row, int(per_head),
+            int(gate == "sigmoid"), self._stream(),
         )
         return out
 
@@ -1490,16 +1522,177 @@ class HipOps:
         )
         return out
 
+    # ---- several residual streams ---------------------------------------------------------------------------
+    def streams_fill(self, x: torch.Tensor, streams: int) -> torch.Tensor:
+        """`streams` copies of x (float32 [T, hidden]) as one tensor [streams, T, hidden]."""
+        self._check(x, "residual stream", torch.float32, (None, None))
+        tokens, hidden = x.shape
+        out = self._empty((int(streams), tokens, hidden), torch.float32)
+        self._call("mlr_streams_fill", self._ptr(x), self._ptr(out), tokens, hidden, int(streams), self._stream())
+        return out
+
+    def streams_step(
+        self,
+        x: torch.Tensor,
+        *,
+        update=None,
+        read_weights: Optional[torch.Tensor] = None,
+        norm_weight: Optional[torch.Tensor] = None,
+        eps: float = 0.0,
+        rows: Optional[torch.Tensor] = None,
+        want_sum: bool = False,
+    ):
+        """One kernel for what happens to residual streams x (float32 [S, T, hidden]) between two sublayers.
+        update = (y, mix [S, S], write [S]): all streams at once from the old ones, x_t = sum_s mix[s, t] x_s +
+        write[t] * y, with y a sublayer's output ([T, hidden] in the engine's dtype or float32, a float32 stack
+        whose sum it is, or a product that has not run).  Then u = sum_s read_weights[s] x_s (None: the plain
+        sum) and, with `norm_weight`, h = u * rsqrt(mean(u^2) + eps) * norm_weight in the engine's dtype.
+        rows: int32 [K] tokens to do this for; the streams themselves are then left as they are.
+        Returns (h or None, u as float32 if `want_sum` else None)."""
+        self._check(x, "residual streams", torch.float32, (None, None, None))
+        streams, tokens, hidden = x.shape
+        y = mix = write = None
+        slices = 0
+        if update is not None:
+            y, mix, write = update
+            y = self.settle(y)
+            if y.dim() == 3:
+                self._check(y, "partial sums", torch.float32, (None, tokens, hidden))
+                slices = y.shape[0]
+            else:
+                self._check(y, "sublayer output", (torch.float32, self.dtype), (tokens, hidden))
+            self._check(mix, "stream mixing matrix", torch.float32, (streams, streams))
+            self._check(write, "stream output weights", torch.float32, (streams,))
+        if read_weights is not None:
+            self._check(read_weights, "stream input weights", torch.float32, (streams,))
+        out_rows = tokens
+        if rows is not None:
+            self._check(rows, "row indices", torch.int32, (None,))
+            out_rows = rows.shape[0]
+        h = total = None
+        if norm_weight is not None:
+            self._check(norm_weight, "norm weight", (torch.float32, self.dtype), (hidden,))
+            h = self._empty((out_rows, hidden), self.dtype)
+        if want_sum:
+            total = self._empty((out_rows, hidden), torch.float32)
+        self._call(
+            "mlr_streams_step", self._ptr(x), streams, tokens, hidden, self._ptr(rows), out_rows, self._ptr(y),
+            int(y is not None and y.dtype == torch.float32), slices, self._ptr(mix), self._ptr(write),
+            self._ptr(read_weights), self._ptr(norm_weight),
+            int(norm_weight is not None and norm_weight.dtype == torch.float32), float(eps), self._ptr(h),
+            self._ptr(total), self.code, self._stream(),
+        )
+        return h, total
+
+    # ---- attention whose heads are normed one by one ---------------------------------------------------------
+    def head_norm_rope_write(
+        self,
+        projected: torch.Tensor,
+        *,
+        heads: int,
+        kv_heads: int,
+        head_dim: int,
+        value_dim: int,
+        kernel_dim: int,
+        eps: float,
+        rotation: Optional[tuple[torch.Tensor, torch.Tensor, int]],
+        slot_mapping: torch.Tensor,
+        key_pages: torch.Tensor,
+        value_pages: torch.Tensor,
+        block_size: int,
+        gated: bool = False,
+        keep_values: bool = False,
+        first_values: Optional[torch.Tensor] = None,
+        mix_weight: Optional[torch.Tensor] = None,
+    ):
+        """From the float32 sums of an attention layer's input product ([T, heads * head_dim + kv_heads * head_dim +
+        kv_heads * value_dim (+ heads)]: queries, keys, values, gate logits) to what the attention kernels take.
+        Queries and keys are rotated (the first r dims of a head in two halves) and then every head is divided
+        by its root mean square over head_dim; every value head by its own over value_dim (eps inside the roots,
+        no weights).  With `first_values` (float32 [T, kv_heads * value_dim]) and `mix_weight` (float32 [1]) the
+        values become (1 - w) v + w first_values.  Queries go to [T, heads * kernel_dim], keys and values into
+        the pages at `slot_mapping`, all zero beyond their own widths.  Returns (queries, sigmoid of the gate
+        logits as float32 [T, heads] or None, the normed values before mixing as float32 if `keep_values`)."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        cos = sin = None
+        rotary = 0
+        if rotation is not None:
+            cos, sin, rotary = rotation
+            self._check(cos, "rotary cos", torch.float32, (tokens, rotary // 2))
+            self._check(sin, "rotary sin", torch.float32, (tokens, rotary // 2))
+        num_pages = self._check_pages(key_pages, value_pages, kv_heads, kernel_dim, block_size)
+        self._check(slot_mapping, "slot mapping", torch.int32, (tokens,))
+        if width < (heads + kv_heads) * head_dim + kv_heads * value_dim + (heads if gated else 0):
+            raise KernelError("the projected rows are too narrow")
+        if first_values is not None:
+            self._check(first_values, "first values", torch.float32, (tokens, kv_heads * value_dim))
+            self._check(mix_weight, "value mixing weight", torch.float32, (1,))
+        q = self._empty((tokens, heads * kernel_dim), self.dtype)
+        gate = self._empty((tokens, heads), torch.float32) if gated else None
+        kept = self._empty((tokens, kv_heads * value_dim), torch.float32) if keep_values else None
+        self._call(
+            "mlr_head_norm_rope_write", self._ptr(projected), width, self._ptr(q), self._ptr(gate), self._ptr(cos),
+            self._ptr(sin), int(rotary), float(eps), self._ptr(slot_mapping), self._ptr(key_pages),
+            self._ptr(value_pages), self._ptr(kept), self._ptr(first_values),
+            self._ptr(mix_weight if first_values is not None else None), self.code, tokens, heads, kv_heads, head_dim,
+            value_dim, kernel_dim, block_size, num_pages, self._stream(),
+        )
+        return q, gate, kept
+
+    # ---- matrix memory with exponential gates -----------------------------------------------------------------
+    def matrix_memory_scan(
+        self,
+        projected: torch.Tensor,
+        state: torch.Tensor,
+        read_rows: torch.Tensor,
+        write_rows: torch.Tensor,
+        ctx: Any,
+        *,
+        heads: int,
+        head_dim: int,
+        value_dim: int,
+        offsets: Sequence[int],
+        cap: float,
+        q_scale: float,
+    ) -> torch.Tensor:
+        """The step's tokens, every entry's in order, through a matrix memory per head: with i = cap tanh(a / cap), f
+        = logsigmoid(cap tanh(b / cap)) (a, b the gates' sums), m' = max(f + m, i), C' = exp(f + m - m') C + exp(i
+        - m') k v^T, n' likewise with k alone, o = C'^T q / (max(|n' . q|, exp(-m')) + 1e-6).  `projected` (float32
+        [T, width]) holds q, k, v and the two gates' sums at the columns `offsets` = (q, k, v, input gate, forget
+        gate); q is scaled by `q_scale`.  state [rows, heads, head_dim * value_dim + head_dim + 1] float32 holds C,
+        n and m of row read_rows[entry] (zeros, m included, where the entry starts its request) and receives them
+        in row write_rows[entry].  Returns o, float32 [T, heads * value_dim]."""
+        self._check(projected, "projected input", torch.float32, (None, None))
+        tokens, width = projected.shape
+        entries = ctx.num_entries
+        self._check(state, "memory state", torch.float32, (None, heads, head_dim * value_dim + head_dim + 1))
+        self._check(read_rows, "state rows to read", torch.int32, (entries,))
+        self._check(write_rows, "state rows to write", torch.int32, (entries,))
+        self._check(ctx.cu_q, "cu_q", torch.int32, (entries + 1,))
+        self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
+        q_off, k_off, v_off, i_off, f_off = (int(o) for o in offsets)
+        out = self._empty((tokens, heads * value_dim), torch.float32)
+        self._call(
+            "mlr_matrix_memory_scan", self._ptr(projected), width, q_off, k_off, v_off, i_off, f_off, self._ptr(state),
+            state.shape[0], self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts),
+            float(cap), float(q_scale), self._ptr(out), entries, heads, head_dim, value_dim, self._stream(),
+        )
+        return out
+
     # ---- routed experts --------------------------------------------------------------------------------
     def route_experts(
         self, logits: torch.Tensor, correction: Optional[torch.Tensor], *, top: int, groups: int, keep_groups: int,
-        scale: float,
+        scale: float, scores: str = "sigmoid", normalise: bool = False,
     ) -> tuple[torch.Tensor, torch.Tensor]:
         """Which experts every token uses (int32 [T, top]) and with what weight (float32 [T, top]),
         from the router's float32 logits z [T, experts]: s = sigmoid(z), c = s + correction; the expert
         axis is cut into `groups` contiguous blocks, a block scores the top-2 sum of its c, and ids are
         the arg-top-`top` of c over the experts of the `keep_groups` highest blocks; weights = s[ids] *
-        `scale` (c only decides)."""
+        `scale` (c only decides).  scores="softmax": s = softmax(z) over all experts instead.  normalise: the
+        chosen weights are divided by their sum (+ 1e-20) before the scale."""
+        if scores not in ("sigmoid", "softmax"):
+            raise KernelError("router scores are 'sigmoid' or 'softmax'")
         self._check(logits, "router logits", torch.float32, (None, None))
         tokens, experts = logits.shape
         if correction is not None:
@@ -1508,7 +1701,8 @@ class HipOps:
         weights = self._empty((tokens, top), torch.float32)
         self._call(
             "mlr_moe_route", self._ptr(logits), self._ptr(correction), self._ptr(ids), self._ptr(weights), tokens,
-            experts, int(top), int(groups), int(keep_groups), float(scale), self._stream(),
+            experts, int(top), int(groups), int(keep_groups), float(scale), int(scores == "softmax"), int(bool(normalise)),
+            self._stream(),
         )
         return ids, weights
 
@@ -1523,17 +1717,22 @@ class HipOps:
         experts: int,
         activation: str,
         kernel: str = "auto",
+        pass_through: int = 0,
     ) -> torch.Tensor:
         """The chosen experts' outputs, weighted: float32 [top, T, hidden] with [j, t] = weights[t, j]
         * down_e(act(up_e(h[t]))), e = ids[t, j]; the sum over j is the mixture's output, which a norm
-        adds to the stream in that order.  up_weight [experts * inner, hidden], down_weight [experts *
+        adds to the stream in that order.  activation "swiglu": a gated expert, up_weight holds every
+        expert's gate rows and then its up rows ([experts * 2 * inner, hidden]) and act is silu(gate) * up, made
+        by a kernel of its own between the two products.  pass_through: ids experts .. experts + pass_through
+        - 1 name experts without matrices whose output is their input: [j, t] = weights[t, j] * h[t].  up_weight [experts * inner, hidden], down_weight [experts *
         hidden, inner].  Three launches: the pairs sorted by expert into tiles of rows, and a grouped
         product over the tiles for each of the two matrices (bfloat16 with hidden and inner multiples
         of 8 on the matrix cores, everything else, and kernel="fma", as plain 32-bit arithmetic)."""
         if kernel not in ("auto", "fma"):
             raise KernelError("kernel must be 'auto' or 'fma'")
-        if activation not in ("relu2", "sigmoid"):
+        if activation not in ("relu2", "sigmoid", "swiglu"):
             raise KernelError(f"unknown activation {activation!r}")
+        gated = activation == "swiglu"
         self._check(h, "expert input", self.dtype, (None, None))
         tokens, hidden = h.shape
         self._check(ids, "expert ids", torch.int32, (tokens, None))
@@ -1541,8 +1740,11 @@ class HipOps:
         self._check(weights, "expert weights", torch.float32, (tokens, top))
         if experts <= 0 or up_weight.shape[0] % experts:
             raise KernelError("the stacked expert matrices do not divide by the number of experts")
-        inner = up_weight.shape[0] // experts
-        self._check(up_weight, "expert up weights", self.dtype, (experts * inner, hidden))
+        wide = up_weight.shape[0] // experts  # rows of an expert's first matrix
+        if gated and wide % 2:
+            raise KernelError("a gated expert's first matrix holds gate rows and as many up rows")
+        inner = wide // 2 if gated else wide
+        self._check(up_weight, "expert up weights", self.dtype, (experts * wide, hidden))
         self._check(down_weight, "expert down weights", self.dtype, (experts * hidden, inner))
         pairs = tokens * top
         mfma = int(kernel == "auto" and self.dtype == torch.bfloat16 and hidden % 8 == 0 and inner % 8 == 0)
@@ -1560,13 +1762,20 @@ class HipOps:
             "mlr_moe_align", self._ptr(ids), pairs, experts, big, max_tiles, self._ptr(order), self._ptr(offsets),
             self._ptr(tiles), self._stream(),
         )
-        act = self._empty((pairs, inner), self.dtype)
+        act = self._empty((pairs, wide), self.dtype)
         out = self._empty((top, tokens, hidden), torch.float32)
         common = (self._ptr(order), self._ptr(offsets), self._ptr(tiles))
         self._call(
             "mlr_moe_gemm", self._ptr(h), self._ptr(up_weight), *common, _VP(None), self._ptr(act), 1, self.code, mfma,
-            max_tiles, tokens, top, inner, hidden, _EPILOGUES[activation], self._stream(),
+            max_tiles, tokens, top, wide, hidden, 0 if gated else _EPILOGUES[activation], self._stream(),
         )
+        if gated:
+            act = self.silu_mul(act)  # rows that no pair owns hold whatever memory held: nothing reads them
+        if pass_through:
+            self._call(
+                "mlr_moe_identity", self._ptr(h), self._ptr(ids), self._ptr(weights), self._ptr(out), self.code, tokens,
+                top, hidden, experts, self._stream(),
+            )
         self._call(
             "mlr_moe_gemm", self._ptr(act), self._ptr(down_weight), *common, self._ptr(weights), self._ptr(out), 0,
             self.code, mfma, max_tiles, tokens, top, hidden, inner, 0, self._stream(),

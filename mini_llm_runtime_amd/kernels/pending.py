@@ -105,3 +105,18 @@ class NormedDelta:
     y: object
     weight: torch.Tensor
     eps: float
+
+
+@dataclass
+class StreamUpdate:
+    """A sublayer's output that enters several residual streams at once: all streams from the old ones,
+    x_t = sum_s mix[s, t] x_s + write[t] * y.  Handed on by arrangements that keep several streams, so that
+    the update and whatever reads the streams next (the next sublayer's weighted sum and norm, the final
+    norm) are one kernel.  `y` is whatever a part may return (see `NormedDelta`)."""
+
+    y: object
+    mix: torch.Tensor
+    write: torch.Tensor
+
+    def as_update(self) -> tuple:
+        return (self.y, self.mix, self.write)

@@ -1,6 +1,6 @@
 """Architectures: each module registers one name with its configuration and builder."""
 
-from . import bubitar, fedolorn, qwen2, vobisun  # noqa: F401  (register Bubitar, Fedolorn, Qwen2ForCausalLM and Vobisun)
+from . import bubitar, fedolorn, pepulix, qwen2, vobisun  # noqa: F401  (register Bubitar, Fedolorn, Pepulix, Qwen2ForCausalLM and Vobisun)
 from .registry import (
     ARCHITECTURES,
     Architecture,

@@ -1,8 +1,8 @@
 """Parts a layer is put together from, and the model that runs them."""
 
 from . import (  # noqa: F401  (register the built-in kinds)
-    attention, block, feed_forward, gated_linear_attention, latent_attention, norm, pooled_attention, position, retention,
-    short_conv, side_by_side, token_input,
+    attention, block, feed_forward, gated_linear_attention, latent_attention, matrix_memory, norm, pooled_attention,
+    position, retention, short_conv, sigmoid_attention, side_by_side, token_input,
 )
 from .base import Block, FeedForward, Mixer, Norm, Part, PositionEncoding
 from .context import KVView, StateView, StepContext

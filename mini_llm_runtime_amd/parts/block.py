@@ -7,7 +7,7 @@ from typing import Mapping, Optional
 import torch
 
 from .base import Block, FeedForward, Mixer, Norm, Part
-from ..kernels.pending import NormedDelta
+from ..kernels.pending import NormedDelta, StreamUpdate
 from ..cache.spec import CompositeSpec
 from .context import StepContext, site_member
 from .registry import register_part
@@ -183,6 +183,79 @@ class ParallelBlock(Block):
             return x, mixed
         ctx.ops.add_(x, mixed)
         return x, self.feed_forward.forward(ctx, h)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Block):
+    """Several residual streams x_1 .. x_S instead of one (`x` is [S, T, hidden], float32).  For each sublayer
+    (the mixer, then the feed-forward) with its own read weights r [S], mixing matrix M [S, S] (indexed [from,
+    to]) and write weights w [S]:
+
+        u = sum_s r[s] x_s;   y = sublayer(norm(u));   x_t <- sum_s M[s, t] x_s + w[t] * y   (all t at once).
+
+    This takes the place of the residual addition.  The update of one sublayer and the weighted sum and norm
+    of the next are one kernel; the last update is handed to the next block (or the model, which sums the
+    streams before its final norm) as a `StreamUpdate`.  A layer may have no feed-forward.
+    """
+
+    replayable = True
+
+    def __init__(
+        self, mixer: Mixer, feed_forward: Optional[FeedForward], norms: Mapping[str, Norm], streams: int = 1
+    ) -> None:
+        needed = ("input", "post_mixer") if feed_forward is not None else ("input",)
+        missing = [n for n in needed if n not in norms]
+        if missing:
+            raise ValueError(f"hyper_connections block needs the norms {needed}, missing {missing}")
+        if streams <= 0 or streams > 16:
+            raise ValueError("hyper_connections keeps 1 to 16 streams")
+        self.streams = int(streams)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norm_input = norms["input"]
+        self.norm_post_mixer = norms["post_mixer"] if feed_forward is not None else None
+        for norm in (self.norm_input, self.norm_post_mixer):
+            if norm is not None and not hasattr(norm, "eps"):
+                raise ValueError("hyper_connections takes RMS norms (a weight and an eps)")
+
+    def children(self) -> dict[str, Part]:
+        parts: dict[str, Part] = {"mixer": self.mixer, "norm_input": self.norm_input}
+        if self.feed_forward is not None:
+            parts.update(feed_forward=self.feed_forward, norm_post_mixer=self.norm_post_mixer)
+        return parts
+
+    def param_specs(self):
+        from .spec import ParamSpec
+
+        S = self.streams
+        specs = {}
+        for name in ("mixer", "ff") if self.feed_forward is not None else ("mixer",):
+            specs[f"{name}_read"] = ParamSpec((S,), init="one_plus_normal", keep_stored_precision=True)
+            specs[f"{name}_write"] = ParamSpec((S,), init="one_plus_normal", keep_stored_precision=True)
+            specs[f"{name}_mix"] = ParamSpec((S, S), init="eye_plus_normal", keep_stored_precision=True)
+        return specs
+
+    def bind(self, params, *, dtype: torch.dtype, device: torch.device) -> None:
+        # the streams and everything that is added into them are 32-bit
+        for name, tensor in params.items():
+            setattr(self, name, tensor.to(torch.float32).contiguous())
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, delta, site: int):
+        ops = ctx.ops
+        if x.dim() != 3 or x.shape[0] != self.streams:
+            raise RuntimeError(f"hyper_connections block of {self.streams} streams was handed a stream of shape {tuple(x.shape)}")
+        owed = delta.as_update() if delta is not None else None
+        h, _ = ops.streams_step(
+            x, update=owed, read_weights=self.mixer_read, norm_weight=self.norm_input.weight, eps=self.norm_input.eps
+        )
+        mixed = self.mixer.forward(ctx, h, site)
+        if self.feed_forward is None:
+            return x, StreamUpdate(mixed, self.mixer_mix, self.mixer_write)
+        h, _ = ops.streams_step(
+            x, update=(mixed, self.mixer_mix, self.mixer_write), read_weights=self.ff_read,
+            norm_weight=self.norm_post_mixer.weight, eps=self.norm_post_mixer.eps,
+        )
+        return x, StreamUpdate(self.feed_forward.forward(ctx, h), self.ff_mix, self.ff_write)
 
 
 def _norm(norm: Norm, consumer: Part, ctx: StepContext, x: torch.Tensor, delta: Optional[torch.Tensor]):

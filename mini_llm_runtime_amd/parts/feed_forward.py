@@ -14,7 +14,8 @@ from .spec import ParamSpec
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
-    """Dense gated feed-forward: `down(silu(gate(x)) * up(x))`, no biases.
+    """Dense gated feed-forward: `down(silu(gate(x)) * up(x))`, without biases or (`bias`) with one on each of
+    the three products; with biases the rows are [Wgate ; Wup] and the gating is a kernel of its own.
 
     Formula: src/mini_llm_runtime/qwen_model_runner.py:215-217.  Gate and up are one
     matrix product over a matrix that holds the rows of Wgate and Wup woven in pairs
@@ -27,28 +28,35 @@ class SwiGLU(FeedForward):
     replayable = True
     takes_pending_norm = True  # `h` goes to the gate/up product only
 
-    def __init__(self, hidden_size: int, intermediate_size: int) -> None:
+    def __init__(self, hidden_size: int, intermediate_size: int, bias: bool = False) -> None:
         if hidden_size <= 0 or intermediate_size <= 0:
             raise ValueError("SwiGLU sizes must be > 0")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
-        self.woven = self.intermediate_size % 2 == 0
+        self.bias = bool(bias)
+        self.woven = self.intermediate_size % 2 == 0 and not self.bias
         self.gate_up_weight: Optional[torch.Tensor] = None
         self.down_weight: Optional[torch.Tensor] = None
+        self.gate_up_bias: Optional[torch.Tensor] = None
+        self.down_bias: Optional[torch.Tensor] = None
 
     def param_specs(self) -> dict[str, ParamSpec]:
-        return {
+        specs = {
             "gate_up_weight": ParamSpec((2 * self.intermediate_size, self.hidden_size)),
             "down_weight": ParamSpec((self.hidden_size, self.intermediate_size)),
         }
+        if self.bias:
+            specs["gate_up_bias"] = ParamSpec((2 * self.intermediate_size,), keep_stored_precision=True)
+            specs["down_bias"] = ParamSpec((self.hidden_size,), keep_stored_precision=True)
+        return specs
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         ops = ctx.ops
         if self.woven:
             hidden = ops.linear(h, self.gate_up_weight, None, swiglu=True)
         else:
-            hidden = ops.silu_mul(ops.linear(h, self.gate_up_weight, None))
-        return ops.linear(hidden, self.down_weight, None, for_stream=True)  # the next norm's delta
+            hidden = ops.silu_mul(ops.linear(h, self.gate_up_weight, self.gate_up_bias))
+        return ops.linear(hidden, self.down_weight, self.down_bias, for_stream=True)  # the next norm's delta
 
 
 @register_part("feed_forward", "clamped_glu")
@@ -98,6 +106,7 @@ class ClampedGLU(FeedForward):
 
 
 ACTIVATIONS = ("relu2", "sigmoid")  # what `ops.linear(..., activation=)` applies to its sums
+EXPERT_ACTIVATIONS = ACTIVATIONS + ("swiglu",)  # an expert may also be gated: down(silu(gate(x)) * up(x))
 
 
 @register_part("feed_forward", "mlp")
@@ -150,6 +159,14 @@ class RoutedExperts(FeedForward):
     outputs, which the next norm adds to the stream in that fixed order.
     Expert matrices are stacked along the rows: up [experts * inner, hidden], down [experts *
     hidden, inner].
+
+    What other routers do differently, each an option:
+    scores: "softmax" makes s the softmax of z over all router outputs instead of sigmoids.
+    normalise: the chosen experts' weights are divided by their sum (+ 1e-20) before `router_scale`.
+    identity: the router has `experts + identity` outputs; the last `identity` of them are experts without
+        matrices whose output is their input itself (times the weight).
+    activation "swiglu": every expert is gated, down_e(silu(gate_e(x)) * up_e(x)); `up_weight` then holds, per
+        expert, its gate rows and then its up rows ([experts * 2 * inner, hidden]).
     """
 
     replayable = True
@@ -164,14 +181,20 @@ class RoutedExperts(FeedForward):
         groups: int = 1,
         keep_groups: int = 1,
         activation: str = "relu2",
+        scores: str = "sigmoid",
+        normalise: bool = False,
+        identity: int = 0,
     ) -> None:
-        if hidden_size <= 0 or intermediate_size <= 0 or experts <= 0 or top <= 0:
+        if hidden_size <= 0 or intermediate_size <= 0 or experts <= 0 or top <= 0 or identity < 0:
             raise ValueError("RoutedExperts sizes must be > 0")
-        if groups <= 0 or experts % groups or not 0 < keep_groups <= groups:
+        routed = experts + identity  # what the router chooses among
+        if groups <= 0 or routed % groups or not 0 < keep_groups <= groups:
             raise ValueError("the experts must divide into equal groups, of which 1..groups are kept")
-        if top > keep_groups * (experts // groups):
+        if top > keep_groups * (routed // groups):
             raise ValueError("the kept groups hold fewer experts than a token uses")
-        if activation not in ACTIVATIONS:
+        if scores not in ("sigmoid", "softmax"):
+            raise ValueError("scores are 'sigmoid' or 'softmax'")
+        if activation not in EXPERT_ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
@@ -181,6 +204,10 @@ class RoutedExperts(FeedForward):
         self.groups = int(groups)
         self.keep_groups = int(keep_groups)
         self.activation = activation
+        self.scores = scores
+        self.normalise = bool(normalise)
+        self.identity = int(identity)
+        self.routed = routed
         self.router_weight: Optional[torch.Tensor] = None
         self.correction: Optional[torch.Tensor] = None
         self.up_weight: Optional[torch.Tensor] = None
@@ -188,9 +215,11 @@ class RoutedExperts(FeedForward):
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {
-            "router_weight": ParamSpec((self.experts, self.hidden_size)),
-            "correction": ParamSpec((self.experts,), keep_stored_precision=True),
-            "up_weight": ParamSpec((self.experts * self.intermediate_size, self.hidden_size)),
+            "router_weight": ParamSpec((self.routed, self.hidden_size)),
+            "correction": ParamSpec((self.routed,), keep_stored_precision=True),
+            "up_weight": ParamSpec(
+                (self.experts * self.intermediate_size * (2 if self.activation == "swiglu" else 1), self.hidden_size)
+            ),
             "down_weight": ParamSpec((self.experts * self.hidden_size, self.intermediate_size)),
         }
 
@@ -204,7 +233,9 @@ class RoutedExperts(FeedForward):
         ids, weights = ops.route_experts(
             logits, self.correction, top=self.top, groups=self.groups, keep_groups=self.keep_groups,
             scale=self.router_scale,
+            **({"scores": self.scores, "normalise": self.normalise} if (self.scores != "sigmoid" or self.normalise) else {}),
         )
         return ops.expert_products(
-            h, self.up_weight, self.down_weight, ids, weights, experts=self.experts, activation=self.activation
+            h, self.up_weight, self.down_weight, ids, weights, experts=self.experts, activation=self.activation,
+            **({"pass_through": self.identity} if self.identity else {}),
         )

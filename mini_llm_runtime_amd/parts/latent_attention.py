@@ -34,6 +34,12 @@ class LatentAttention(Mixer):
     side by side in the matrix cores' columns), and Wuv is applied once per token to the attended
     latent.  The pages hold c twice: as part of the key row and, transposed, as the value.
 
+    q_rank: the queries go through a latent of their own: c_q = rmsnorm(Wdq h) * w_q (32-bit), q = Wuq c_q.  The
+    input product then has Wdq's rows in a product of its own, whose normed result feeds the query product.
+
+    A rotation that pairs neighbouring dims (`interleaved`) is served by reordering, once, the rows that make
+    the rotated parts of queries and key (a dot product does not care in which order both list their dims).
+
     kv_source: True for a site that reads an earlier site's cache (`OrderEntry.reads_cache_of`): it
     has no Wdkv and writes nothing; its cache spec equals the owner's.
     """
@@ -54,6 +60,7 @@ class LatentAttention(Mixer):
         reads_cache: bool = False,
         sink: bool = True,
         output_gate: bool = True,
+        q_rank: Optional[int] = None,
     ) -> None:
         if min(hidden_size, num_heads, head_dim, rot_dim, value_dim, kv_rank) <= 0:
             raise ValueError("LatentAttention sizes must be > 0")
@@ -70,6 +77,9 @@ class LatentAttention(Mixer):
         self.reads_cache = bool(reads_cache)
         self.has_sink = bool(sink)
         self.output_gate = bool(output_gate)
+        if q_rank is not None and q_rank <= 0:
+            raise ValueError("q_rank must be > 0 or None")
+        self.q_rank = None if q_rank is None else int(q_rank)
         # the one head size that the attention kernels and the pages see: a cached row [c ; r], padded
         self.kernel_dim = -(-(self.kv_rank + self.rot_dim) // 16) * 16
         # rows of up to 256 run on the matrix cores (in bfloat16); wider ones, up to 1,024, the plain kernel
@@ -83,6 +93,9 @@ class LatentAttention(Mixer):
         self.uv_weight: Optional[torch.Tensor] = None
         self.sink: Optional[torch.Tensor] = None
         self.o_weight: Optional[torch.Tensor] = None
+        self.dq_weight: Optional[torch.Tensor] = None
+        self.q_norm_weight: Optional[torch.Tensor] = None
+        self.uq_weight: Optional[torch.Tensor] = None
 
     # rows of the one input product: queries, then (unless the cache is another site's) latent and
     # rotated key part, then the gate
@@ -99,8 +112,9 @@ class LatentAttention(Mixer):
         return self.num_heads if self.output_gate else 0
 
     def param_specs(self) -> dict[str, ParamSpec]:
+        own_q = 0 if self.q_rank is not None else self.q_rows
         specs = {
-            "in_weight": ParamSpec((self.q_rows + self.kv_rows + self.gate_rows, self.hidden_size)),
+            "in_weight": ParamSpec((own_q + self.kv_rows + self.gate_rows, self.hidden_size)),
             "uk_weight": ParamSpec((self.num_heads * self.head_dim, self.kv_rank)),
             "uv_weight": ParamSpec((self.num_heads * self.value_dim, self.kv_rank)),
             "o_weight": ParamSpec((self.hidden_size, self.num_heads * self.value_dim)),
@@ -109,6 +123,12 @@ class LatentAttention(Mixer):
             specs["latent_norm_weight"] = ParamSpec((self.kv_rank,), init="one_plus_normal", keep_stored_precision=True)
         if self.has_sink:
             specs["sink"] = ParamSpec((self.num_heads,), keep_stored_precision=True)
+        if self.q_rank is not None:
+            specs["dq_weight"] = ParamSpec((self.q_rank, self.hidden_size))
+            specs["q_norm_weight"] = ParamSpec((self.q_rank,), init="one_plus_normal", keep_stored_precision=True)
+            specs["uq_weight"] = ParamSpec((self.q_rows, self.q_rank))
+        if self.q_rank is not None and self.kv_rows + self.gate_rows == 0:
+            del specs["in_weight"]  # a site that reads another's cache, ungated: nothing but queries to project
         return specs
 
     def bind(self, params, *, dtype: torch.dtype, device: torch.device) -> None:
@@ -120,6 +140,18 @@ class LatentAttention(Mixer):
         self.uv = self.uv_weight.view(self.num_heads, self.value_dim, self.kv_rank)
         if self.sink is not None:
             self.sink = self.sink.to(torch.float32)
+        order = self.position.half_split_order() if self.position is not None else None
+        if order is not None and order != list(range(len(order))):
+            # neighbouring pairs -> halves: the rows of every head's rotated query part, and of the key part
+            index = torch.tensor(order, device=device)
+            qd = self.head_dim + self.rot_dim
+            q_matrix = self.uq_weight if self.q_rank is not None else self.in_weight
+            for head in range(self.num_heads):
+                at = head * qd + self.head_dim
+                q_matrix[at : at + self.rot_dim] = q_matrix[at : at + self.rot_dim][index]
+            if not self.reads_cache:
+                at = (0 if self.q_rank is not None else self.q_rows) + self.kv_rank
+                self.in_weight[at : at + self.rot_dim] = self.in_weight[at : at + self.rot_dim][index]
 
     def children(self) -> dict[str, Part]:
         return {"position": self.position} if self.position is not None else {}
@@ -138,7 +170,16 @@ class LatentAttention(Mixer):
             raise RuntimeError("a latent-attention site owns its cache exactly when it has a down-projection of its own")
         rotation = self.position.rotation(ctx) if self.position is not None else None
         # the input product's sums stay 32-bit: the latent's norm, the rotation and the gate read them unrounded
-        projected = ops.linear(h, self.in_weight, None, out_dtype=torch.float32)
+        queries = None
+        if self.q_rank is not None:
+            latent = ops.rmsnorm(
+                ops.linear(h, self.dq_weight, None, out_dtype=torch.float32), self.q_norm_weight, self.norm_eps
+            )
+            queries = ops.linear(latent, self.uq_weight, None, out_dtype=torch.float32)
+        if self.in_weight is not None:
+            projected = ops.linear(h, self.in_weight, None, out_dtype=torch.float32)
+        else:
+            projected = queries
         q_plain, q_latent, gate = ops.latent_prepare(
             projected,
             heads=self.num_heads,
@@ -155,6 +196,7 @@ class LatentAttention(Mixer):
             value_pages=cache.value,
             block_size=cache.block_size,
             kernel_dim=self.kernel_dim,
+            **({"queries": queries} if queries is not None else {}),
         )
         if cache.writable:
             cache.written()
@@ -177,5 +219,7 @@ class LatentAttention(Mixer):
             **({"sinks": self.sink} if self.sink is not None else {}),
         )
         # the attended latent of every head through its Wuv, times the head's gate
-        merged = ops.heads_linear(attended, self.uv, in_stride=self.kernel_dim, row_scale=gate)
+        merged = ops.heads_linear(
+            attended, self.uv, in_stride=self.kernel_dim, **({"row_scale": gate} if gate is not None else {})
+        )
         return ops.linear(merged, self.o_weight, None, for_stream=True)

@@ -17,7 +17,7 @@ from .registry import build_part
 from .spec import LayerSpec, ModelSpec, ParamSpec, PartSpec
 
 
-def _build_layer(spec: LayerSpec) -> Block:
+def _build_layer(spec: LayerSpec, streams: int = 0) -> Block:
     mixer = build_part("mixer", spec.mixer)
     feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
     norms = {name: build_part("norm", s) for name, s in spec.norms.items()}
@@ -26,6 +26,8 @@ def _build_layer(spec: LayerSpec) -> Block:
         extra["token_input"] = build_part("token_input", spec.token_input)
     if spec.mixer_filter is not None:
         extra["mixer_filter"] = build_part("input_filter", spec.mixer_filter)
+    if streams:  # only arrangements that keep several streams are told how many
+        extra["streams"] = streams
     return build_part("block", PartSpec(spec.block), mixer=mixer, feed_forward=feed_forward, norms=norms, **extra)
 
 
@@ -38,7 +40,7 @@ def _walk(prefix: str, part: Part) -> Iterator[tuple[str, Part]]:
 class DecoderModel:
     def __init__(self, spec: ModelSpec) -> None:
         self.spec = spec
-        self.layers: list[Block] = [_build_layer(s) for s in spec.layers]
+        self.layers: list[Block] = [_build_layer(s, spec.residual_streams) for s in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm)
         self.position_embedding = (
             build_part("position", spec.position_embedding) if spec.position_embedding is not None else None
@@ -159,11 +161,17 @@ class DecoderModel:
             ops.scale_softcap_(x, spec.embedding_scale)
         if self.position_embedding is not None:
             ops.add_(x, self.position_embedding.embed(ctx))
+        streams = spec.residual_streams
+        if streams:
+            x = ops.streams_fill(x, streams)  # [S, T, hidden]; the blocks hand on their last update un-applied
         delta: Optional[torch.Tensor] = None
         capture = site_outputs is not None and logit_rows is not None and logit_rows.numel() > 0
         for site, entry in enumerate(self.spec.order):
             x, delta = self.layers[entry.layer].forward(ctx, x, delta, site)
-            if capture:
+            if capture and streams:
+                owed = delta.as_update() if delta is not None else None
+                site_outputs.append(ops.streams_step(x, update=owed, rows=logit_rows, want_sum=True)[1])
+            elif capture:
                 # the site's own output is not added into the stream yet: add it here, in 32-bit
                 rows = ops.gather_rows(x, logit_rows)
                 if delta is not None:
@@ -173,6 +181,16 @@ class DecoderModel:
                 site_outputs.append(rows)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
+        if streams:
+            # the sum of the streams behind the last update, normed: one kernel, on the wanted rows only
+            h, _ = ops.streams_step(
+                x, update=delta.as_update() if delta is not None else None, rows=logit_rows,
+                norm_weight=self.final_norm.weight, eps=self.final_norm.eps,
+            )
+            logits = ops.linear(h, self.head_weight, self.head_bias, out_dtype=torch.float32)
+            if spec.logit_scale != 1.0 or spec.logit_softcap is not None:
+                ops.scale_softcap_(logits, spec.logit_scale, spec.logit_softcap)
+            return logits
         if ctx.logits_for_all:
             rows, delta_rows = x, delta
         else:

@@ -14,8 +14,8 @@ from typing import Any, Mapping, Optional
 class ParamSpec:
     """One parameter tensor of a part.
 
-    init: "normal" (N(0, std)) or "one_plus_normal" (1 + N(0, std)); used by the
-        random-weights mode only.
+    init: "normal" (N(0, std)), "one_plus_normal" (1 + N(0, std)) or, for a square matrix,
+        "eye_plus_normal" (identity + N(0, std)); used by the random-weights mode only.
     keep_stored_precision: a vector (norm weight, bias) that a checkpoint stores in
         32-bit stays 32-bit in the bfloat16 engine; matrices always take the
         engine's dtype.
@@ -155,3 +155,6 @@ class ModelSpec:
     head_bias: bool = False  # logits += parameter `head.bias`
     logit_scale: float = 1.0  # logits times this ...
     logit_softcap: Optional[float] = None  # ... then cap * tanh(logits / cap)
+    # > 0: the residual stream is that many streams [S, T, hidden], all equal to the embedded tokens at the
+    # start and summed before the final norm; every layer's arrangement then is one that keeps streams
+    residual_streams: int = 0

@@ -128,17 +128,22 @@ def expected_tensors(model: DecoderModel) -> dict[str, tuple[WeightRule, tuple[i
 
 
 def _check_coverage(model: DecoderModel) -> None:
-    """Every row of every parameter must be fed by exactly one rule."""
+    """Every row of every parameter must be fed by exactly one rule (a parameter that is one number counts
+    as one row)."""
     specs = model.param_specs()
     covered: dict[str, list[int]] = {name: [] for name in specs}
+
+    def row_count(name: str) -> int:
+        return specs[name].shape[0] if specs[name].shape else 1
+
     for rule in model.spec.weight_rules:
         if rule.must_equal is not None:
             continue
-        rows = specs[rule.dest].shape[0]
+        rows = row_count(rule.dest)
         n = rows if rule.rows is None else rule.rows
         covered[rule.dest].extend(rule.dest_rows(n))
     for name, rows in covered.items():
-        if sorted(rows) != list(range(specs[name].shape[0])):
+        if sorted(rows) != list(range(row_count(name))):
             raise ValueError(f"the weight rules do not fill every row of {name} exactly once")
 
 
@@ -203,6 +208,9 @@ def load_weights(
                     continue
                 tensor = rule.take(stored)
                 dest = params[rule.dest]
+                if dest.dim() == 0:  # one number
+                    dest.copy_(tensor.to(dest.dtype))
+                    continue
                 rows = dest.shape[0] if rule.rows is None else rule.rows
                 if rule.block:
                     index = torch.tensor(rule.dest_rows(rows), dtype=torch.long, device=dest.device)

@@ -36,6 +36,8 @@ def random_tensor(name: str, shape: tuple[int, ...], spec: ParamSpec, seed: int,
     values = torch.randn(shape, generator=_generator(seed, name), dtype=torch.float32) * std
     if spec.init == "one_plus_normal":
         values += 1.0
+    elif spec.init == "eye_plus_normal":
+        values += torch.eye(shape[0], shape[1])
     elif spec.init != "normal":
         raise ValueError(f"unknown init {spec.init!r} for {name}")
     return values.to(dtype)
@@ -115,6 +117,8 @@ def bind_random_weights(
         t.normal_(0.0, std, generator=g)
         if spec.init == "one_plus_normal":
             t += 1.0
+        elif spec.init == "eye_plus_normal":
+            t += torch.eye(spec.shape[0], spec.shape[1], dtype=kind, device=device)
         elif spec.init != "normal":
             raise ValueError(f"unknown init {spec.init!r} for {name}")
         params[name] = t

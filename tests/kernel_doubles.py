@@ -137,13 +137,17 @@ class TorchOps:
 
     def latent_prepare(
         self, projected, *, heads, head_dim, rot_dim, kv_rank, own_cache, gated, norm_weight, eps, rotation, slot_mapping,
-        key_pages, value_pages, block_size, kernel_dim,
+        key_pages, value_pages, block_size, kernel_dim, queries=None,
     ):
         self._count("latent_prepare")
         tokens = projected.shape[0]
         p = projected.float()
-        q = p[:, : heads * (head_dim + rot_dim)].view(tokens, heads, head_dim + rot_dim)
-        at = heads * (head_dim + rot_dim)
+        if queries is not None:  # the query sums come from a product of their own
+            q = queries.float().view(tokens, heads, head_dim + rot_dim)
+            at = 0
+        else:
+            q = p[:, : heads * (head_dim + rot_dim)].view(tokens, heads, head_dim + rot_dim)
+            at = heads * (head_dim + rot_dim)
         q_plain = q[..., :head_dim].reshape(tokens, heads * head_dim).to(self.dtype)
         q_latent = torch.zeros(tokens, heads, kernel_dim, dtype=torch.float32)
         q_latent[..., kv_rank : kv_rank + rot_dim] = self._rotate(q[..., head_dim:], rotation)
@@ -200,16 +204,18 @@ class TorchOps:
         return out.view(tokens, heads * value_dim)
 
     def retention_gate(
-        self, retained, projected, *, heads, value_dim, gate_offset, eps, norm_weight=None, scale=1.0, out=None, column=0
+        self, retained, projected, *, heads, value_dim, gate_offset, eps, norm_weight=None, scale=1.0, out=None, column=0,
+        gate="silu",
     ):
         self._count("retention_gate")
         tokens = retained.shape[0]
         o = retained.float().view(tokens, heads, value_dim)
         o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
-        if norm_weight is not None:
-            o = o * norm_weight.float()
+        if norm_weight is not None:  # one weight for all heads, or one over all heads side by side
+            o = o * (norm_weight.float().view(heads, value_dim) if norm_weight.numel() == heads * value_dim else norm_weight.float())
         z = projected[:, gate_offset : gate_offset + heads * value_dim].float()
-        y = (o.reshape(tokens, heads * value_dim) * (z * torch.sigmoid(z)) * scale).to(self.dtype)
+        act = torch.sigmoid(z) if gate == "sigmoid" else z * torch.sigmoid(z)
+        y = (o.reshape(tokens, heads * value_dim) * act * scale).to(self.dtype)
         if out is None:
             return y
         out[:, column : column + heads * value_dim] = y
@@ -359,7 +365,7 @@ class TorchOps:
 
     def paged_attention(
         self, qkv, key_pages, value_pages, block_table, ctx, *, num_heads, num_kv_heads, head_dim, block_size, scale, window,
-        defer_merge=False, plan=None, chunk=None, sinks=None, pooled=None,
+        defer_merge=False, plan=None, chunk=None, sinks=None, pooled=None, score_bias=None,
     ):
         self._count("paged_attention")
         tokens = qkv.shape[0]
@@ -388,7 +394,9 @@ class TorchOps:
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)
             s = torch.einsum("hd,nhd->hn", q[t], k) * scale
-            if sinks is not None:  # one more term of the denominator, with no key and no value
+            if score_bias is not None:  # no softmax: every key weighs by itself
+                w = torch.sigmoid(s + score_bias.float()[:, None])
+            elif sinks is not None:  # one more term of the denominator, with no key and no value
                 top = torch.maximum(s.max(-1).values, sinks.float())
                 e = torch.exp(s - top[:, None])
                 w = e / (e.sum(-1) + torch.exp(sinks.float() - top))[:, None]
@@ -397,11 +405,99 @@ class TorchOps:
             out[t] = torch.einsum("hn,nhd->hd", w, v)
         return out.reshape(tokens, num_heads * head_dim).to(self.dtype)
 
+    # several residual streams ---------------------------------------------------------------------
+    def streams_fill(self, x, streams):
+        self._count("streams_fill")
+        return x.float()[None].repeat(streams, 1, 1).contiguous()
+
+    def streams_step(self, x, *, update=None, read_weights=None, norm_weight=None, eps=0.0, rows=None, want_sum=False):
+        self._count("streams_step")
+        assert x.dtype == torch.float32 and x.dim() == 3
+        new = x
+        if update is not None:
+            y, mix, write = update
+            y = self._sum(self.settle(y))
+            new = torch.einsum("st,snw->tnw", mix.float(), x) + write.float()[:, None, None] * y[None]
+            if rows is None:
+                x.copy_(new)
+        if rows is not None:
+            new = new[:, rows.long()]
+        u = new.sum(0) if read_weights is None else torch.einsum("s,snw->nw", read_weights.float(), new)
+        h = None
+        if norm_weight is not None:
+            h = (norm_weight.float() * (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps))).to(self.dtype)
+        return h, (u if want_sum else None)
+
+    def head_norm_rope_write(
+        self, projected, *, heads, kv_heads, head_dim, value_dim, kernel_dim, eps, rotation, slot_mapping, key_pages,
+        value_pages, block_size, gated=False, keep_values=False, first_values=None, mix_weight=None,
+    ):
+        self._count("head_norm_rope_write")
+        tokens = projected.shape[0]
+        p = projected.float()
+        a, b = heads * head_dim, (heads + kv_heads) * head_dim
+        c = b + kv_heads * value_dim
+
+        def unit(x):
+            return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+        q = unit(self._rotate(p[:, :a].view(tokens, heads, head_dim), rotation))
+        k = unit(self._rotate(p[:, a:b].view(tokens, kv_heads, head_dim), rotation))
+        v = unit(p[:, b:c].view(tokens, kv_heads, value_dim))
+        kept = v.reshape(tokens, kv_heads * value_dim).clone() if keep_values else None
+        if first_values is not None:
+            w = mix_weight.float()[0]
+            v = (1.0 - w) * v + w * first_values.float().view(tokens, kv_heads, value_dim)
+        q_out = torch.zeros(tokens, heads, kernel_dim)
+        q_out[..., :head_dim] = q
+        k_row = torch.zeros(tokens, kv_heads, kernel_dim)
+        k_row[..., :head_dim] = k
+        v_row = torch.zeros(tokens, kv_heads, kernel_dim)
+        v_row[..., :value_dim] = v
+        slots = slot_mapping.long()
+        ok = slots >= 0
+        page, off = slots[ok] // block_size, slots[ok] % block_size
+        key_pages[page, :, off, :] = k_row[ok].to(key_pages.dtype)
+        value_pages[page, :, :, off] = v_row[ok].to(value_pages.dtype)
+        gate = torch.sigmoid(p[:, c : c + heads]) if gated else None
+        return q_out.view(tokens, heads * kernel_dim).to(self.dtype), gate, kept
+
+    def matrix_memory_scan(
+        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, offsets, cap, q_scale
+    ):
+        self._count("matrix_memory_scan")
+        tokens = projected.shape[0]
+        p = projected.float()
+        qa, ka, va, ia, fa = offsets
+        q = p[:, qa : qa + heads * head_dim].view(tokens, heads, head_dim) * q_scale
+        k = p[:, ka : ka + heads * head_dim].view(tokens, heads, head_dim)
+        v = p[:, va : va + heads * value_dim].view(tokens, heads, value_dim)
+        gi = cap * torch.tanh(p[:, ia : ia + heads] / cap)
+        gf = torch.nn.functional.logsigmoid(cap * torch.tanh(p[:, fa : fa + heads] / cap))
+        out = torch.zeros(tokens, heads, value_dim, dtype=torch.float32)
+        cells = head_dim * value_dim
+        for r in range(ctx.num_entries):
+            a, b = int(ctx.cu_q[r]), int(ctx.cu_q[r + 1])
+            row = state[int(read_rows[r])].float().clone() if int(ctx.q_starts[r]) > 0 else torch.zeros_like(state[0])
+            C = row[:, :cells].reshape(heads, head_dim, value_dim)
+            n = row[:, cells : cells + head_dim].clone()
+            m = row[:, cells + head_dim].clone()
+            for t in range(a, b):
+                m_new = torch.maximum(gf[t] + m, gi[t])
+                keep, take = torch.exp(gf[t] + m - m_new), torch.exp(gi[t] - m_new)
+                C = keep[:, None, None] * C + take[:, None, None] * k[t][:, :, None] * v[t][:, None, :]
+                n = keep[:, None] * n + take[:, None] * k[t]
+                m = m_new
+                below = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+                out[t] = torch.einsum("hdv,hd->hv", C, q[t]) / below[:, None]
+            state[int(write_rows[r])] = torch.cat([C.reshape(heads, cells), n, m[:, None]], dim=1)
+        return out.view(tokens, heads * value_dim)
+
     # routed experts ------------------------------------------------------------------------------
-    def route_experts(self, logits, correction, *, top, groups, keep_groups, scale):
+    def route_experts(self, logits, correction, *, top, groups, keep_groups, scale, scores="sigmoid", normalise=False):
         self._count("route_experts")
         tokens, experts = logits.shape
-        s = torch.sigmoid(logits.float())
+        s = torch.softmax(logits.float(), -1) if scores == "softmax" else torch.sigmoid(logits.float())
         c = s + correction.float()
         per = experts // groups
         ids = torch.empty(tokens, top, dtype=torch.int32)
@@ -411,12 +507,13 @@ class TorchOps:
             kept = sorted(range(groups), key=lambda g: (-score[g], g))[:keep_groups]
             allowed = [e for e in range(experts) if e // per in kept]
             chosen = sorted(allowed, key=lambda e: (-float(c[t, e]), e))[:top]
+            total = sum(float(s[t, e]) for e in chosen) + 1e-20 if normalise else 1.0
             for j, e in enumerate(chosen):
                 ids[t, j] = e
-                weights[t, j] = s[t, e] * scale
+                weights[t, j] = s[t, e] / total * scale
         return ids.to(logits.device), weights.to(logits.device)
 
-    def expert_products(self, h, up_weight, down_weight, ids, weights, *, experts, activation):
+    def expert_products(self, h, up_weight, down_weight, ids, weights, *, experts, activation, pass_through=0):
         self._count("expert_products")
         tokens, hidden = h.shape
         top = ids.shape[1]
@@ -426,8 +523,17 @@ class TorchOps:
         for t in range(tokens):
             for j in range(top):
                 e = int(ids[t, j])
+                if e >= experts:  # an expert without matrices: its input itself
+                    assert e < experts + pass_through
+                    out[j, t] = weights[t, j] * h[t].float()
+                    continue
                 z = up[e] @ h[t].float()
-                a = torch.clamp(z, min=0.0) ** 2 if activation == "relu2" else torch.sigmoid(z)
+                if activation == "swiglu":
+                    z = z.to(self.dtype).float()
+                    half = z.shape[0] // 2
+                    a = z[:half] * torch.sigmoid(z[:half]) * z[half:]
+                else:
+                    a = torch.clamp(z, min=0.0) ** 2 if activation == "relu2" else torch.sigmoid(z)
                 out[j, t] = weights[t, j] * (down[e] @ a.to(self.dtype).float())
         return out
 
