@@ -153,7 +153,7 @@ def write_safetensors(
                     f"the header expects {name!r} {dtype} {shape}"
                 )
             data = tensor.detach().cpu().contiguous()
-            f.write(data.view(torch.uint8).numpy().tobytes() if data.numel() else b"")
+            f.write(data.reshape(-1).view(torch.uint8).numpy().tobytes() if data.numel() else b"")
 
 
 def save_state_dict(path: str | Path, tensors: dict[str, torch.Tensor]) -> None:
