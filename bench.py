@@ -803,6 +803,31 @@ class Bench:
                 pairs = sum(min(t + 1, a.window) + max(0, t - a.window + 1) // a.pool for t in range(tokens))
                 flops += 2 * tokens * per_token + 2 * a.heads * (a.dim + a.vdim) * pairs
             return flops
+        if getattr(config, "architecture", "") == "Pepulix":
+            # per layer: the mixer's products (latent attention as the kernels run it: the query's two products,
+            # the query through Wuk^T, scores and values over rows of kv_rank + rot_dim and kv_rank, the attended
+            # latent through Wuv; the memory's state update and read, 2 x dim x vdim a head and token), the
+            # feed-forward (a token's `top` experts counted as gated experts, and the router)
+            for layer in config.layers:
+                a, m = layer.mixer, layer.mlp
+                pairs = tokens * (tokens + 1) // 2
+                if a.kind == "attention":
+                    per_token = width * (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim) + a.heads) + a.heads * a.vdim * width
+                    per_pair = a.heads * (a.dim + a.vdim)
+                elif a.kind == "latent_attention":
+                    per_token = width * (a.q_rank + a.kv_rank + a.rot_dim) + a.q_rank * a.heads * (a.dim + a.rot_dim)
+                    per_token += a.heads * a.kv_rank * (a.dim + a.vdim) + a.heads * a.vdim * width
+                    per_pair = a.heads * (2 * a.kv_rank + a.rot_dim)
+                else:
+                    per_token = width * (2 * a.heads * a.dim + 2 * a.heads * a.vdim + 2 * a.heads) + a.heads * a.vdim * width
+                    per_token += 2 * a.heads * a.dim * a.vdim
+                    per_pair = 0
+                if m is not None and m.kind == "moe":
+                    per_token += 3 * width * m.ff * m.top + width * (m.experts + m.identity)
+                elif m is not None:
+                    per_token += 3 * width * m.ff
+                flops += 2 * tokens * per_token + 2 * per_pair * pairs
+            return flops
         if hasattr(config, "token_side_dim"):
             # retention: four input products, the state update and read (2 x dim x vdim a head and token, as the
             # recurrence counts them), the output product; latent attention as the kernels run it: input

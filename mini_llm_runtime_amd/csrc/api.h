@@ -278,7 +278,10 @@ int mlr_head_norm_rope_write(const float* projected, int width, void* q_out, flo
 int mlr_matrix_memory_scan(const float* projected, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
                            float* state, int state_rows, const int* read_rows, const int* write_rows, const int* cu_q,
                            const int* q_starts, float cap, float q_scale, float* out, int entries, int heads, int dim,
-                           int vdim, hipStream_t stream);
+                           int vdim, int tokens, float* runs, float* run_gates, hipStream_t stream);
+// runs (or null: every entry is walked whole): float32 [mlr_matrix_memory_runs(tokens, entries), heads, dim * vdim + dim
+// + 1] and run_gates [that many, heads, 2] of scratch; entries are then walked in runs of 64 tokens, all at once.
+int mlr_matrix_memory_runs(int tokens, int entries);
 
 // tokens[k] = argmax(logits[k, :]) (first maximum), or, where temperature[k] > 0,
 // the first index whose cumulative exp((x - max) / temperature) exceeds

@@ -176,7 +176,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ cu_q, const int* __restrict__ context_lens, bf16* __restrict__ out,
     float* __restrict__ partial, int heads, int kv_heads, int head_tiles, int block_size, int num_pages,
-    float scale, int window, int chunk, int part, int splits, const float* __restrict__ sinks, int keep_partial) {
+    float scale, int window, int chunk, int part, int splits, const float* __restrict__ sinks, int keep_partial,
+    const float* __restrict__ score_bias) {
   __shared__ float sm_acc[kDecodeWaves][16][D];
   __shared__ float sm_m[kDecodeWaves][16];
   __shared__ float sm_l[kDecodeWaves][16];
@@ -226,6 +227,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   // Per tile: scores of both halves, ONE softmax update, one 32-key value product per 16 dims.
   constexpr int kStride = kDecodeWaves * 32;
   const float scale2 = scale * 1.44269504088896340736f;
+  // score_bias: no softmax.  A visible key weighs sigmoid(score * scale + bias of the head) whatever the other
+  // keys are; the state's maximum stays 0 (so every merge weighs all shares alike) and nothing is divided.
+  const bool gated = score_bias != nullptr;
+  const float bias2 = gated ? score_bias[head_ok ? head : 0] * 1.44269504088896340736f : 0.f;
   for (int ts0 = kb + wave * 32; ts0 < ke; ts0 += kDecodeDepth * kStride) {
     DecodeTilePages pages[kDecodeDepth];
 #pragma unroll
@@ -260,22 +265,32 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
           tmax = fmaxf(tmax, sc[half][i]);
         }
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-      const float m_new = fmaxf(sm.m, tmax * scale2);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
-      const float alpha = fast_exp2(sm.m - m_use);
-      float sum = 0.f;
       float pr[2][4];
+      float alpha = 1.0f;
+      if (gated) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pr[half][i] = fast_exp2(fmaf(sc[half][i], scale2, -m_use));
-          sum += pr[half][i];
-        }
-      sm.l = sm.l * alpha + sum;
-      sm.m = m_new;
+          for (int i = 0; i < 4; ++i)  // a hidden score is -inf: 1 / (1 + 2^inf) = 0
+            pr[half][i] = __builtin_amdgcn_rcpf(1.0f + fast_exp2(-fmaf(sc[half][i], scale2, bias2)));
+        sm.m = 0.f;
+      } else {
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(sm.m, tmax * scale2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a column that has seen no key yet
+        alpha = fast_exp2(sm.m - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            pr[half][i] = fast_exp2(fmaf(sc[half][i], scale2, -m_use));
+            sum += pr[half][i];
+          }
+        sm.l = sm.l * alpha + sum;
+        sm.m = m_new;
+      }
       if (__any(alpha != 1.0f)) {
 #pragma unroll
         for (int dt = 0; dt < kDimTiles; ++dt)
@@ -327,7 +342,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const int h = kvh * group + htile * 16 + c;
     if (splits == 1 && !keep_partial) {
       num *= join_sink(sinks, h, mstar, den);  // with partitions the merge does this, once
-      const float v = poisoned ? __builtin_nanf("") : num / den;
+      const float v = poisoned ? __builtin_nanf("") : (gated ? num : num / den);
       out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(v);
     } else {
       float* dst = partial + ((static_cast<int64_t>(entry) * heads + h) * splits + split) * kPartialStride;
@@ -351,7 +366,7 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
                                                                   bf16* __restrict__ out, int heads, int window,
                                                                   int chunk, int part, int all_splits,
                                                                   const float* __restrict__ sinks,
-                                                                  const float* __restrict__ extra) {
+                                                                  const float* __restrict__ extra, int gated) {
   const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -430,7 +445,8 @@ __global__ __launch_bounds__(kWave) void attn_decode_merge_kernel(const float* _
 #pragma unroll
   for (int j = 0; j < (D + kWave - 1) / kWave; ++j) {
     const int d = lane + j * kWave;
-    if (d < D) out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(num[j] * keep / den);
+    // gated: shares of keys that weigh by themselves (all maxima 0): their plain sum
+    if (d < D) out[(static_cast<int64_t>(t) * heads + h) * D + d] = f32_to_bf16(gated ? num[j] : num[j] * keep / den);
   }
 }
 
@@ -488,7 +504,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     const bf16* __restrict__ value_pages, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ cu_q, const int* __restrict__ context_lens,
     bf16* __restrict__ out, int num_tiles, int heads, int kv_heads, int bs_shift, int num_pages, float scale,
-    int window, int chunk, float* __restrict__ partial, const float* __restrict__ sinks, int keep_partial) {
+    int window, int chunk, float* __restrict__ partial, const float* __restrict__ sinks, int keep_partial,
+    const float* __restrict__ score_bias) {
   // gridDim.y > 1: the keys of every tile are cut into that many runs, one workgroup each, which
   // leave their unnormalised results in `partial` for attn_prefill_merge (few tiles behind a long
   // context would otherwise be as many long chains on a few compute units).
@@ -574,6 +591,8 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
   const int w_max_first = first_visible_key(pos0 + q0 + wave * kWaveQ + kWaveQ - 1, window, chunk);
   // softmax in base 2: exp(x) = exp2(x * log2(e))
   const float scale2 = scale * 1.44269504088896340736f;
+  const bool gated = score_bias != nullptr;  // keys that weigh by themselves, see attn_decode_kernel
+  const float bias2 = gated ? score_bias[head] * 1.44269504088896340736f : 0.f;
 
   float m_run[QB], l_run[QB];  // l: this lane's share of the sum
   f32x4_t acc[QB][kDimTiles];
@@ -741,6 +760,22 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
             }
       }
       uint32_t pw[QB][kSubTiles][2];
+      if (gated) {
+        // no softmax: every key weighs sigmoid(score * scale + bias) by itself (hidden: -inf gives 0), the
+        // state's maximum stays 0 and nothing is rescaled
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+#pragma unroll
+          for (int sub = 0; sub < kSubTiles; ++sub) {
+            float p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = __builtin_amdgcn_rcpf(1.0f + fast_exp2(-fmaf(s[b][sub][i], scale2, bias2)));
+            pw[b][sub][0] = pack_bf16x2(p[0], p[1]);
+            pw[b][sub][1] = pack_bf16x2(p[2], p[3]);
+          }
+          m_run[b] = 0.f;
+        }
+      } else
 #pragma unroll
       for (int b = 0; b < QB; ++b) {
         float tmax = -INFINITY;
@@ -861,7 +896,7 @@ __global__ __launch_bounds__(256 * kKeyGroups) void attn_prefill_kernel(
     }
     if (q_ok[b]) {
       const float keep = join_sink(sinks, head, m_run[b], l);
-      const float inv = keep / l;
+      const float inv = gated ? 1.0f : keep / l;
       bf16* orow = out + (static_cast<int64_t>(t_first + qi[b]) * heads + head) * D;
 #pragma unroll
       for (int dt = 0; dt < kDimTiles; ++dt) {
@@ -883,7 +918,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
                                                                  const int* __restrict__ cu_q,
                                                                  bf16* __restrict__ out, int heads, int splits,
                                                                  int tile_q, const float* __restrict__ sinks,
-                                                                 const float* __restrict__ extra) {
+                                                                 const float* __restrict__ extra, int gated) {
   const int tile = blockIdx.x / heads;
   const int head = blockIdx.x - tile * heads;
   const int entry = tiles[2 * tile];
@@ -922,8 +957,8 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
     }
     const float keep = join_sink(sinks, head, mstar, den);
     bf16* orow = out + (static_cast<int64_t>(t_first + q0 + qq) * heads + head) * D;
-    orow[d] = f32_to_bf16(num0 * keep / den);
-    orow[d + 1] = f32_to_bf16(num1 * keep / den);
+    orow[d] = f32_to_bf16(gated ? num0 : num0 * keep / den);
+    orow[d + 1] = f32_to_bf16(gated ? num1 : num1 * keep / den);
   }
 }
 
@@ -957,8 +992,10 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
                          const int* block_table, int table_width, const int* cu_q, const int* context_lens,
                          void* out, float* partial, int entries, int heads, int kv_heads, int block_size,
                          int num_pages, float scale, int window, int chunk, int part, int splits, int merge,
-                         const float* sinks, const float* extra, hipStream_t stream) {
+                         const float* sinks, const float* extra, const float* score_bias, hipStream_t stream) {
   MLR_REQUIRE(q && key_pages && value_pages && block_table && cu_q && context_lens && out, "null pointer");
+  MLR_REQUIRE(score_bias == nullptr || (sinks == nullptr && extra == nullptr && merge),
+              "keys weighed one by one have no sink and no share made elsewhere, and are merged here");
   MLR_REQUIRE(entries > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "bad head counts");
   MLR_REQUIRE(block_size > 0 && block_size % 4 == 0, "block_size must be a multiple of 4");
   MLR_REQUIRE(num_pages > 0 && table_width > 0, "page sizes must be > 0");
@@ -985,7 +1022,7 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
 #define MLR_DECODE(depth)                                                                                       \
   attn_decode_kernel<depth><<<grid, kDecodeWaves * kWave, 0, stream>>>(                                         \
       qp, q_stride, kp, vp, block_table, table_width, cu_q, context_lens, op, partial, heads, kv_heads,         \
-      head_tiles, block_size, num_pages, scale, window, chunk, part, splits, sinks, keep_partial)
+      head_tiles, block_size, num_pages, scale, window, chunk, part, splits, sinks, keep_partial, score_bias)
   bool launched = false;
   if constexpr (kMaxDecodeDepth >= 4) {
     if (tiles_per_wave >= 4) {
@@ -1005,7 +1042,8 @@ int mlr_attention_decode(const void* q, int64_t q_stride, const void* key_pages,
   MLR_REQUIRE(sinks == nullptr || merge, "partitions left unmerged cannot carry sinks");
   if ((splits > 1 || keep_partial) && merge) {
     attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(
-        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, extra);
+        partial, cu_q, context_lens, static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, extra,
+        score_bias != nullptr);
     MLR_LAUNCH_CHECK();
   }
   return 0;
@@ -1020,7 +1058,7 @@ int mlr_attention_decode_merge(const float* partial, const int* cu_q, const int*
   MLR_REQUIRE(entries > 0 && heads > 0 && heads <= 65535, "bad sizes");
   MLR_REQUIRE(part > 0 && part % 64 == 0 && splits > 1 && window >= 0 && chunk >= 0, "bad partitions");
   attn_decode_merge_kernel<<<dim3(entries, heads), kWave, 0, stream>>>(partial, cu_q, context_lens,
-                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, nullptr);
+                                                                      static_cast<bf16*>(out), heads, window, chunk, part, splits, sinks, nullptr, 0);
   MLR_LAUNCH_CHECK();
   return 0;
 }
@@ -1046,8 +1084,11 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
                           const int* block_table, int table_width, const int* tiles, int num_tiles, int wide,
                           const int* cu_q, const int* context_lens, void* out, int heads, int kv_heads,
                           int block_size, int num_pages, float scale, int window, int chunk, int splits,
-                          float* partial, const float* sinks, const float* extra, hipStream_t stream) {
+                          float* partial, const float* sinks, const float* extra, const float* score_bias,
+                          hipStream_t stream) {
   MLR_REQUIRE(splits >= 1 && splits <= 64, "splits must lie within 1..64");
+  MLR_REQUIRE(score_bias == nullptr || (sinks == nullptr && extra == nullptr),
+              "keys weighed one by one have no sink and no share made elsewhere");
   MLR_REQUIRE((splits == 1 && extra == nullptr) || partial != nullptr, "several key runs, or a share made elsewhere, need scratch memory");
   const int keep_partial = extra != nullptr;
   MLR_REQUIRE(q && key_pages && value_pages && block_table && tiles && cu_q && context_lens && out, "null pointer");
@@ -1092,13 +1133,13 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
           static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
-          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial);  \
+          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial, score_bias);  \
     else                                                                                                      \
       attn_prefill_kernel<qb, false><<<grid, 256 * kKeyGroups, kPrefillLds, stream>>>(                        \
           static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(key_pages),                         \
           static_cast<const bf16*>(value_pages), block_table, table_width, tiles, cu_q, context_lens,         \
           static_cast<bf16*>(out), num_tiles, heads, kv_heads, bs_shift, num_pages, scale, window, chunk, partial,  \
-          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial);  \
+          (splits > 1 || keep_partial) ? nullptr : sinks, keep_partial, score_bias);  \
   } while (0)
   if constexpr (D <= 128) {
     if (wide)
@@ -1113,7 +1154,7 @@ int mlr_attention_prefill(const void* q, int64_t q_stride, const void* key_pages
   if (splits > 1 || keep_partial) {
     const int tile_q = (wide && D <= 128) ? 2 * kTileQ : kTileQ;
     attn_prefill_merge_kernel<<<dim3(static_cast<unsigned>(num_tiles) * heads), 256, 0, stream>>>(
-        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q, sinks, extra);
+        partial, tiles, cu_q, static_cast<bf16*>(out), heads, splits, tile_q, sinks, extra, score_bias != nullptr);
     MLR_LAUNCH_CHECK();
   }
   return 0;

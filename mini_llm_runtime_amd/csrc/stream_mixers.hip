@@ -173,21 +173,47 @@ __global__ __launch_bounds__(256) void head_norm_rope_write_kernel(
 // column c of C and the same rows of n; eight tokens' q and k at a time go through LDS, rows beyond dim as zeros,
 // so the inner loops have no conditions.
 constexpr int kMemTokens = 8;
+constexpr int kMemRun = 64;  // tokens of a run when long entries are walked in runs
+
+// Long entries are cut into runs of kMemRun tokens, all runs of all entries walked at once, twice.  With F the
+// sum of a run's f and the run walked from nothing (C = n = 0, m = -inf), its own sums U (of C and n alike) and
+// maximum m_u relate the states before and after it:  m' = max(F + m, m_u),  X' = exp(F + m - m') X + exp(m_u -
+// m') U.  kRunSums makes U, m_u and F of every run; matrix_memory_carry_kernel walks an entry's runs element by
+// element and leaves the state BEFORE every run where its U was (and the entry's last state in its row);
+// kRunScan walks every run again from that state and writes the outputs.
+enum MemoryMode : int { kWholeEntries = 0, kRunSums = 1, kRunScan = 2 };
+
+// Which entry run number `run` (counted over all entries in order) belongs to, and its tokens.
+__device__ inline bool find_memory_run(const int* __restrict__ cu_q, int entries, int run, int& entry, int& t_begin,
+                                       int& t_end) {
+  int at = 0;
+  for (int e = 0; e < entries; ++e) {
+    const int a = cu_q[e], b = cu_q[e + 1];
+    const int runs = (b - a + kMemRun - 1) / kMemRun;
+    if (run < at + runs) {
+      entry = e;
+      t_begin = a + (run - at) * kMemRun;
+      t_end = min(t_begin + kMemRun, b);
+      return true;
+    }
+    at += runs;
+  }
+  return false;
+}
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int R>  // rows of the state a lane holds: dim <= 4 * R
+template <int R, int MODE>  // R: rows of the state a lane holds, dim <= 4 * R
 __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
     const float* __restrict__ p, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
     float* __restrict__ state, const int* __restrict__ read_rows, const int* __restrict__ write_rows,
     const int* __restrict__ cu_q, const int* __restrict__ q_starts, float cap, float q_scale, float* __restrict__ out,
-    int heads, int dim, int vdim) {
+    int heads, int dim, int vdim, int entries, float* __restrict__ runs, float* __restrict__ run_gates) {
   constexpr int MAXD = 4 * R;
   __shared__ __attribute__((aligned(16))) float sq[kMemTokens][MAXD];
   __shared__ __attribute__((aligned(16))) float sk[kMemTokens][MAXD];
   __shared__ float sv[kMemTokens][64];
   __shared__ float sg[kMemTokens][2];
-  const int entry = blockIdx.x;
   const int h = blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
@@ -196,12 +222,22 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
   const int c_local = wave * 16 + lane % 16;
   const int col = blockIdx.z * 64 + c_local;
   const bool col_ok = col < vdim;
-  const int t_begin = cu_q[entry];
-  const int t_end = cu_q[entry + 1];
   const int64_t per_head = static_cast<int64_t>(dim) * vdim + dim + 1;
-  const bool fresh = q_starts[entry] == 0;
-  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * per_head;
-  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * per_head;
+  int entry = blockIdx.x, t_begin, t_end;
+  bool fresh;
+  const float* src;
+  float* dst;
+  if constexpr (MODE == kWholeEntries) {
+    t_begin = cu_q[entry];
+    t_end = cu_q[entry + 1];
+    fresh = q_starts[entry] == 0;
+    src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * per_head;
+    dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * per_head;
+  } else {
+    if (!find_memory_run(cu_q, entries, blockIdx.x, entry, t_begin, t_end)) return;  // the grid is sized for the most runs
+    fresh = MODE == kRunSums;
+    src = dst = runs + (static_cast<int64_t>(blockIdx.x) * heads + h) * per_head;
+  }
 
   float C[R], n[R];
 #pragma unroll
@@ -211,7 +247,8 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
     C[j] = (in && col_ok) ? src[static_cast<int64_t>(r) * vdim + col] : 0.f;
     n[j] = in ? src[static_cast<int64_t>(dim) * vdim + r] : 0.f;
   }
-  float m = fresh ? 0.f : src[static_cast<int64_t>(dim) * vdim + dim];
+  float m = fresh ? (MODE == kRunSums ? -INFINITY : 0.f) : src[static_cast<int64_t>(dim) * vdim + dim];
+  float f_sum = 0.f;
 
   for (int t0 = t_begin; t0 < t_end; t0 += kMemTokens) {
     const int nb = min(kMemTokens, t_end - t0);
@@ -238,9 +275,10 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
       const float ig = sg[tt][0];
       const float fg = sg[tt][1];
       const float m_new = fmaxf(fg + m, ig);
-      const float keep = expf(fg + m - m_new);
+      const float keep = expf(fg + m - m_new);  // exp(-inf) = 0 where a run starts from nothing
       const float take = expf(ig - m_new);
       m = m_new;
+      f_sum += fg;
       const float v = sv[tt][c_local] * take;
       float num = 0.f, nq = 0.f;
 #pragma unroll
@@ -249,15 +287,26 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
         const float qv = sq[tt][g + 4 * j];
         C[j] = fmaf(keep, C[j], kv * v);
         n[j] = fmaf(keep, n[j], kv * take);
-        num = fmaf(C[j], qv, num);
-        nq = fmaf(n[j], qv, nq);
+        if constexpr (MODE != kRunSums) {
+          num = fmaf(C[j], qv, num);
+          nq = fmaf(n[j], qv, nq);
+        }
       }
-      num += __shfl_xor(num, 16, kWave);
-      num += __shfl_xor(num, 32, kWave);
-      nq += __shfl_xor(nq, 16, kWave);
-      nq += __shfl_xor(nq, 32, kWave);
-      if (g == 0 && col_ok)
-        out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+      if constexpr (MODE != kRunSums) {
+        num += __shfl_xor(num, 16, kWave);
+        num += __shfl_xor(num, 32, kWave);
+        nq += __shfl_xor(nq, 16, kWave);
+        nq += __shfl_xor(nq, 32, kWave);
+        if (g == 0 && col_ok)
+          out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+      }
+    }
+  }
+  if constexpr (MODE == kRunScan) return;  // the carry has left the entry's last state in its row
+  if constexpr (MODE == kRunSums) {
+    if (blockIdx.z == 0 && tid == 0) {
+      run_gates[(static_cast<int64_t>(blockIdx.x) * heads + h) * 2] = f_sum;
+      run_gates[(static_cast<int64_t>(blockIdx.x) * heads + h) * 2 + 1] = m;
     }
   }
 #pragma unroll
@@ -268,7 +317,42 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
       if (blockIdx.z == 0 && wave == 0 && lane % 16 == 0) dst[static_cast<int64_t>(dim) * vdim + r] = n[j];
     }
   }
-  if (blockIdx.z == 0 && tid == 0) dst[static_cast<int64_t>(dim) * vdim + dim] = m;
+  if (MODE == kWholeEntries && blockIdx.z == 0 && tid == 0) dst[static_cast<int64_t>(dim) * vdim + dim] = m;
+}
+
+// One thread per element of a head's C and n: walks its entry's runs in order (see kMemRun above).
+__global__ __launch_bounds__(256) void matrix_memory_carry_kernel(
+    float* __restrict__ runs, const float* __restrict__ run_gates, float* __restrict__ state,
+    const int* __restrict__ read_rows, const int* __restrict__ write_rows, const int* __restrict__ cu_q,
+    const int* __restrict__ q_starts, int heads, int dim, int vdim) {
+  const int entry = blockIdx.x;
+  const int h = blockIdx.y;
+  const int elem = blockIdx.z * 256 + threadIdx.x;
+  const int cells = dim * vdim + dim;  // C and n; m sits behind them
+  if (elem >= cells) return;
+  const int64_t per_head = cells + 1;
+  int first_run = 0;
+  for (int e = 0; e < entry; ++e) first_run += (cu_q[e + 1] - cu_q[e] + kMemRun - 1) / kMemRun;
+  const int count = (cu_q[entry + 1] - cu_q[entry] + kMemRun - 1) / kMemRun;
+  const bool fresh = q_starts[entry] == 0;
+  const float* src = state + (static_cast<int64_t>(read_rows[entry]) * heads + h) * per_head;
+  float x = fresh ? 0.f : src[elem];
+  float m = fresh ? 0.f : src[cells];
+  for (int r = 0; r < count; ++r) {
+    const int64_t at = static_cast<int64_t>(first_run + r) * heads + h;
+    float* slot = runs + at * per_head;
+    const float u = slot[elem];
+    const float f_sum = run_gates[at * 2];
+    const float m_u = run_gates[at * 2 + 1];
+    slot[elem] = x;
+    if (elem == 0) slot[cells] = m;
+    const float m_new = fmaxf(f_sum + m, m_u);
+    x = expf(f_sum + m - m_new) * x + expf(m_u - m_new) * u;
+    m = m_new;
+  }
+  float* dst = state + (static_cast<int64_t>(write_rows[entry]) * heads + h) * per_head;
+  dst[elem] = x;
+  if (elem == 0) dst[cells] = m;
 }
 
 }  // namespace mlr
@@ -337,11 +421,15 @@ int mlr_head_norm_rope_write(const float* projected, int width, void* q_out, flo
   return 0;
 }
 
+// The most runs that `tokens` tokens in `entries` entries make (every entry may end in a run that is not full).
+int mlr_matrix_memory_runs(int tokens, int entries) { return tokens / kMemRun + entries; }
+
 int mlr_matrix_memory_scan(const float* projected, int width, int q_off, int k_off, int v_off, int i_off, int f_off,
                            float* state, int state_rows, const int* read_rows, const int* write_rows, const int* cu_q,
                            const int* q_starts, float cap, float q_scale, float* out, int entries, int heads, int dim,
-                           int vdim, hipStream_t stream) {
+                           int vdim, int tokens, float* runs, float* run_gates, hipStream_t stream) {
   MLR_REQUIRE(projected && state && read_rows && write_rows && cu_q && q_starts && out, "null pointer");
+  MLR_REQUIRE((runs == nullptr) == (run_gates == nullptr) && (runs == nullptr || tokens > 0), "runs come with their gates' sums");
   MLR_REQUIRE(entries > 0 && heads > 0 && heads < 65536 && dim > 0 && vdim > 0 && state_rows > 0, "sizes must be > 0");
   MLR_REQUIRE(dim <= 256, "heads of up to 256 dims");
   MLR_REQUIRE(cap > 0.f, "the gates' cap must be > 0");
@@ -349,19 +437,34 @@ int mlr_matrix_memory_scan(const float* projected, int width, int q_off, int k_o
                   k_off + heads * dim <= width && v_off + heads * vdim <= width && i_off + heads <= width &&
                   f_off + heads <= width,
               "the projected rows do not hold what the offsets name");
-  const dim3 grid(entries, heads, (vdim + 63) / 64);
-#define MLR_MEMORY(R)                                                                                               \
-  matrix_memory_scan_kernel<R><<<grid, 256, 0, stream>>>(projected, width, q_off, k_off, v_off, i_off, f_off, state, \
-                                                         read_rows, write_rows, cu_q, q_starts, cap, q_scale, out,   \
-                                                         heads, dim, vdim)
-  if (dim <= 64)
-    MLR_MEMORY(16);
-  else if (dim <= 128)
-    MLR_MEMORY(32);
-  else
-    MLR_MEMORY(64);
-#undef MLR_MEMORY
+#define MLR_MEMORY(R, MODE, FIRST)                                                                                \
+  matrix_memory_scan_kernel<R, MODE><<<dim3(FIRST, heads, (vdim + 63) / 64), 256, 0, stream>>>(                    \
+      projected, width, q_off, k_off, v_off, i_off, f_off, state, read_rows, write_rows, cu_q, q_starts, cap,     \
+      q_scale, out, heads, dim, vdim, entries, runs, run_gates)
+#define MLR_MEMORY_SIZED(MODE, FIRST) \
+  do {                                \
+    if (dim <= 64)                    \
+      MLR_MEMORY(16, MODE, FIRST);    \
+    else if (dim <= 128)              \
+      MLR_MEMORY(32, MODE, FIRST);    \
+    else                              \
+      MLR_MEMORY(64, MODE, FIRST);    \
+  } while (0)
+  if (runs == nullptr) {
+    MLR_MEMORY_SIZED(kWholeEntries, entries);
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
+  const int most = mlr_matrix_memory_runs(tokens, entries);
+  MLR_MEMORY_SIZED(kRunSums, most);
   MLR_LAUNCH_CHECK();
+  matrix_memory_carry_kernel<<<dim3(entries, heads, (dim * vdim + dim + 255) / 256), 256, 0, stream>>>(
+      runs, run_gates, state, read_rows, write_rows, cu_q, q_starts, heads, dim, vdim);
+  MLR_LAUNCH_CHECK();
+  MLR_MEMORY_SIZED(kRunScan, most);
+  MLR_LAUNCH_CHECK();
+#undef MLR_MEMORY_SIZED
+#undef MLR_MEMORY
   return 0;
 }
 

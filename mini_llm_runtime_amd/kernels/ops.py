@@ -42,8 +42,9 @@ _SIGNATURES = {
         [_VP, _I, _VP, _VP, _VP, _VP, _I, _F, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP], _I,
     ),
     "mlr_matrix_memory_scan": (
-        [_VP, _I, _I, _I, _I, _I, _I, _VP, _I, _VP, _VP, _VP, _VP, _F, _F, _VP, _I, _I, _I, _I, _VP], _I,
+        [_VP, _I, _I, _I, _I, _I, _I, _VP, _I, _VP, _VP, _VP, _VP, _F, _F, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP], _I,
     ),
+    "mlr_matrix_memory_runs": ([_I, _I], _I),
     "mlr_moe_identity": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_heads_linear": ([_VP, _I64, _I, _VP, _VP, _I64, _I, _VP, _I, _I, _I, _I, _I, _VP], _I),
     "mlr_retention_scan": (
@@ -108,13 +109,13 @@ _SIGNATURES = {
     "mlr_attention_wide_tile": ([], _I),
     "mlr_attention_decode_scratch": ([_I, _I, _I], _I64),
     "mlr_attention_decode": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP],
         _I,
     ),
     "mlr_attention_decode_merge": ([_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP], _I),
     "mlr_attention_prefill_scratch": ([_I, _I, _I, _I], _I64),
     "mlr_attention_prefill": (
-        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP, _VP, _VP],
+        [_VP, _I64, _VP, _VP, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _I, _I, _VP, _VP, _VP, _VP, _VP],
         _I,
     ),
 }
@@ -984,7 +985,6 @@ class HipOps:
             and 16 <= head_dim <= 256
             and block_size % 4 == 0
             and stride % 8 == 0
-            and score_bias is None
         )
         num_tiles = int(getattr(plan, "num_query_tiles", 0))
         num_decode = int(getattr(plan, "num_decode_entries", 0))
@@ -1038,13 +1038,14 @@ class HipOps:
             leave_unmerged = (
                 defer_merge and self.tuning.fuse_merge and not num_tiles and num_decode == entries == tokens
                 and 1 < splits <= 64 and tokens <= self.FUSED_TOKENS and not chunk and sinks is None and share is None
+                and score_bias is None
             )
             self._call(
                 "mlr_attention_decode", self._ptr(qkv), stride, self._ptr(key_pages), self._ptr(value_pages),
                 self._ptr(block_table), width, self._ptr(ctx.cu_q), self._ptr(ctx.context_lens), self._ptr(out),
                 self._ptr(partial), entries, num_heads, num_kv_heads, block_size, num_pages, float(scale),
                 int(window or 0), chunk, part, splits, int(not leave_unmerged), self._ptr(sinks), self._ptr(share),
-                self._stream(), lib=lib,
+                self._ptr(score_bias), self._stream(), lib=lib,
             )
             if leave_unmerged:
                 return PendingMerge(
@@ -1082,7 +1083,7 @@ class HipOps:
                 self._ptr(block_table), width, self._ptr(tiles), num_tiles, wide, self._ptr(ctx.cu_q),
                 self._ptr(ctx.context_lens), self._ptr(out), num_heads, num_kv_heads, block_size, num_pages,
                 float(scale), int(window or 0), chunk, key_runs, self._ptr(partial), self._ptr(sinks), self._ptr(share),
-                self._stream(), lib=lib,
+                self._ptr(score_bias), self._stream(), lib=lib,
             )
         return out
 
@@ -1641,6 +1642,8 @@ class HipOps:
         return q, gate, kept
 
     # ---- matrix memory with exponential gates -----------------------------------------------------------------
+    MEMORY_RUNS_FROM = 128  # tokens more than entries from which the memory's scan walks runs instead of whole entries
+
     def matrix_memory_scan(
         self,
         projected: torch.Tensor,
@@ -1655,6 +1658,7 @@ class HipOps:
         offsets: Sequence[int],
         cap: float,
         q_scale: float,
+        in_runs: Optional[bool] = None,
     ) -> torch.Tensor:
         """The step's tokens, every entry's in order, through a matrix memory per head: with i = cap tanh(a / cap), f
         = logsigmoid(cap tanh(b / cap)) (a, b the gates' sums), m' = max(f + m, i), C' = exp(f + m - m') C + exp(i
@@ -1662,7 +1666,10 @@ class HipOps:
         [T, width]) holds q, k, v and the two gates' sums at the columns `offsets` = (q, k, v, input gate, forget
         gate); q is scaled by `q_scale`.  state [rows, heads, head_dim * value_dim + head_dim + 1] float32 holds C,
         n and m of row read_rows[entry] (zeros, m included, where the entry starts its request) and receives them
-        in row write_rows[entry].  Returns o, float32 [T, heads * value_dim]."""
+        in row write_rows[entry].  Returns o, float32 [T, heads * value_dim].  Steps of few tokens an entry walk
+        every entry whole; steps with `MEMORY_RUNS_FROM` tokens more than entries cut them into runs of 64 tokens
+        that are all walked at once, twice, with the state carried between the walks (`in_runs` forces one way):
+        that reorders 32-bit sums only."""
         self._check(projected, "projected input", torch.float32, (None, None))
         tokens, width = projected.shape
         entries = ctx.num_entries
@@ -1673,10 +1680,18 @@ class HipOps:
         self._check(ctx.q_starts, "q_starts", torch.int32, (entries,))
         q_off, k_off, v_off, i_off, f_off = (int(o) for o in offsets)
         out = self._empty((tokens, heads * value_dim), torch.float32)
+        if in_runs is None:
+            in_runs = tokens >= entries + self.MEMORY_RUNS_FROM
+        runs = gates = None
+        if in_runs:
+            most = int(self.lib.mlr_matrix_memory_runs(tokens, entries))
+            runs = self._empty((most, heads, head_dim * value_dim + head_dim + 1), torch.float32)
+            gates = self._empty((most, heads, 2), torch.float32)
         self._call(
             "mlr_matrix_memory_scan", self._ptr(projected), width, q_off, k_off, v_off, i_off, f_off, self._ptr(state),
             state.shape[0], self._ptr(read_rows), self._ptr(write_rows), self._ptr(ctx.cu_q), self._ptr(ctx.q_starts),
-            float(cap), float(q_scale), self._ptr(out), entries, heads, head_dim, value_dim, self._stream(),
+            float(cap), float(q_scale), self._ptr(out), entries, heads, head_dim, value_dim, tokens, self._ptr(runs),
+            self._ptr(gates), self._stream(),
         )
         return out
 

@@ -463,7 +463,8 @@ class TorchOps:
         return q_out.view(tokens, heads * kernel_dim).to(self.dtype), gate, kept
 
     def matrix_memory_scan(
-        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, offsets, cap, q_scale
+        self, projected, state, read_rows, write_rows, ctx, *, heads, head_dim, value_dim, offsets, cap, q_scale,
+        in_runs=None,
     ):
         self._count("matrix_memory_scan")
         tokens = projected.shape[0]

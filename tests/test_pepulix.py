@@ -397,9 +397,10 @@ def _step_context(lengths, starts, ops):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("in_runs", [False, True], ids=["whole", "in-runs"])
 @pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 32), (3, 20, 12), (4, 64, 48), (1, 128, 70), (2, 200, 20), (1, 1, 1)])
-def test_memory_scan_and_its_state_rows(heads, dim, vdim):
-    """Entries of 1, 5 and 150 tokens, one that starts its request on a row full of NaN, two that go on from a
+def test_memory_scan_and_its_state_rows(heads, dim, vdim, in_runs):
+    """Entries of 1, 5 and 150 tokens (three runs, the last not full), one that starts its request on a row full of NaN, two that go on from a
     carried state; rows that no entry writes stay as they were.  Against the stand-in's loop over tokens, which
     the CPU tests hold against the plain implementation."""
     hip, double = _ops("hip", torch.float32), TorchOps(torch.float32, "cpu")
@@ -423,7 +424,7 @@ def test_memory_scan_and_its_state_rows(heads, dim, vdim):
     got_state = state.cuda()
     got = hip.matrix_memory_scan(
         projected.cuda(), got_state, read.cuda(), write.cuda(), _step_context(lengths, starts, hip), heads=heads,
-        head_dim=dim, value_dim=vdim, offsets=offsets, cap=6.0, q_scale=dim**-0.5,
+        head_dim=dim, value_dim=vdim, offsets=offsets, cap=6.0, q_scale=dim**-0.5, in_runs=in_runs,
     )
     torch.testing.assert_close(got.cpu(), want, rtol=2e-4, atol=2e-4)
     torch.testing.assert_close(got_state.cpu(), want_state, rtol=2e-4, atol=2e-4, equal_nan=True)
