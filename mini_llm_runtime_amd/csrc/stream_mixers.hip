@@ -80,6 +80,105 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
   }
 }
 
+// The same for up to four streams and rows of up to 4,096 numbers that are a multiple of four: a thread owns groups
+// of four neighbouring columns (16-byte loads and stores), all of its loads are asked for before the first is
+// used, and its sums u stay in registers between the row's sum of squares and the normed result, so every
+// number is read once.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kStreamGroups = 4;  // groups of four columns a thread owns: 256 * 4 * 4 columns a row at most
+
+template <typename T, int S>
+__global__ __launch_bounds__(256) void streams_step_rows_kernel(
+    float* __restrict__ x, int tokens, int width, const int* __restrict__ rows, const void* __restrict__ y,
+    int y_is_f32, int slices, const float* __restrict__ mix, const float* __restrict__ out_w,
+    const float* __restrict__ in_w, const void* __restrict__ norm_w, int norm_is_f32, float eps, T* __restrict__ h_out,
+    float* __restrict__ sum_out) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int64_t t = rows != nullptr ? rows[r] : r;
+  const bool write_back = rows == nullptr;
+  const int64_t plane = static_cast<int64_t>(tokens) * width;
+  float w_mix[S][S], w_out[S], w_in[S];  // uniform: scalar registers
+#pragma unroll
+  for (int a = 0; a < S; ++a) {
+#pragma unroll
+    for (int b = 0; b < S; ++b) w_mix[a][b] = mix != nullptr ? mix[a * S + b] : 0.f;
+    w_out[a] = out_w != nullptr ? out_w[a] : 0.f;
+    w_in[a] = in_w != nullptr ? in_w[a] : 1.f;
+  }
+  f32x4 xs[kStreamGroups][S], yv[kStreamGroups];
+#pragma unroll
+  for (int i = 0; i < kStreamGroups; ++i) {
+    const int c = (threadIdx.x + i * 256) * 4;
+    const bool in = c < width;
+    const int64_t at = t * width + (in ? c : 0);
+#pragma unroll
+    for (int a = 0; a < S; ++a) xs[i][a] = in ? *reinterpret_cast<const f32x4*>(x + a * plane + at) : f32x4{0.f, 0.f, 0.f, 0.f};
+    yv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (y != nullptr && in) {
+      if (slices > 0) {
+        for (int k = 0; k < slices; ++k) yv[i] += *reinterpret_cast<const f32x4*>(static_cast<const float*>(y) + k * plane + at);
+      } else if (y_is_f32) {
+        yv[i] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(y) + at);
+      } else {
+        typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+        const u16x4 raw = *reinterpret_cast<const u16x4*>(static_cast<const bf16*>(y) + at);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[i][e] = to_f32(bf16{raw[e]});
+      }
+    }
+  }
+  f32x4 us[kStreamGroups];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kStreamGroups; ++i) {
+    const int c = (threadIdx.x + i * 256) * 4;
+    const bool in = c < width;
+    f32x4 u = {0.f, 0.f, 0.f, 0.f};
+    if (y != nullptr) {
+#pragma unroll
+      for (int to = 0; to < S; ++to) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int a = 0; a < S; ++a)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = fmaf(w_mix[a][to], xs[i][a][e], v[e]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = fmaf(w_out[to], yv[i][e], v[e]);
+          u[e] = fmaf(w_in[to], v[e], u[e]);
+        }
+        if (write_back && in) *reinterpret_cast<f32x4*>(x + to * plane + t * width + c) = v;
+      }
+    } else {
+#pragma unroll
+      for (int a = 0; a < S; ++a)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[e] = fmaf(w_in[a], xs[i][a][e], u[e]);
+    }
+    us[i] = u;
+    ss += (u[0] * u[0] + u[1] * u[1]) + (u[2] * u[2] + u[3] * u[3]);
+    if (sum_out != nullptr && in) *reinterpret_cast<f32x4*>(sum_out + static_cast<int64_t>(r) * width + c) = u;
+  }
+  if (h_out == nullptr) return;
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(width) + eps);
+#pragma unroll
+  for (int i = 0; i < kStreamGroups; ++i) {
+    const int c = (threadIdx.x + i * 256) * 4;
+    if (c >= width) continue;
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = us[i][e] * inv * load_as_f32(norm_w, c + e, norm_is_f32);
+    T* dst = h_out + static_cast<int64_t>(r) * width + c;
+    if constexpr (sizeof(T) == 4) {
+      *reinterpret_cast<f32x4*>(dst) = f32x4{o[0], o[1], o[2], o[3]};
+    } else {
+      typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+      *reinterpret_cast<u16x4*>(dst) = u16x4{f32_to_bf16(o[0]).bits, f32_to_bf16(o[1]).bits, f32_to_bf16(o[2]).bits, f32_to_bf16(o[3]).bits};
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void streams_fill_kernel(const float* __restrict__ x, float* __restrict__ out,
                                                            int64_t plane, int streams) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -381,6 +480,31 @@ int mlr_streams_step(float* x, int streams, int tokens, int width, const int* ro
   MLR_REQUIRE(slices >= 0 && (slices == 0 || (y && y_is_f32)), "partial sums are float32");
   MLR_REQUIRE(h_out == nullptr || norm_w, "normed activations need a norm weight");
   MLR_REQUIRE(dtype == kF32 || dtype == kBF16, "dtype must be 0 (float32) or 1 (bfloat16)");
+  if (streams <= 4 && width % 4 == 0 && width <= 256 * 4 * kStreamGroups) {
+#define MLR_STREAMS(T, S)                                                                                          \
+  streams_step_rows_kernel<T, S><<<out_rows, 256, 0, stream>>>(x, tokens, width, rows, y, y_is_f32, slices, mix, out_w, \
+                                                               in_w, norm_w, norm_is_f32, eps, static_cast<T*>(h_out), \
+                                                               sum_out)
+#define MLR_STREAMS_OF(T)   \
+  do {                      \
+    if (streams == 1)       \
+      MLR_STREAMS(T, 1);    \
+    else if (streams == 2)  \
+      MLR_STREAMS(T, 2);    \
+    else if (streams == 3)  \
+      MLR_STREAMS(T, 3);    \
+    else                    \
+      MLR_STREAMS(T, 4);    \
+  } while (0)
+    if (dtype == kF32)
+      MLR_STREAMS_OF(float);
+    else
+      MLR_STREAMS_OF(bf16);
+#undef MLR_STREAMS_OF
+#undef MLR_STREAMS
+    MLR_LAUNCH_CHECK();
+    return 0;
+  }
   if (dtype == kF32)
     streams_step_kernel<float><<<out_rows, 256, 0, stream>>>(x, streams, tokens, width, rows, y, y_is_f32, slices, mix,
                                                              out_w, in_w, norm_w, norm_is_f32, eps,
