@@ -1,0 +1,110 @@
+"""Drawn Pepulix configurations: every size, constant, layer order and option drawn anew, random weights, a drawn
+schedule and page size, the engine against the plain implementation.  A model of this design that nobody has
+looked at must run without a change of code; this is the nearest a test gets.
+
+float32: 1e-3 of the logits' size (chosen models stay below 1e-4; drawn ones of five layers with several streams
+are more often ill-conditioned).  bfloat16: the bounds of `test_pepulix._compare` (all rows together, single
+rows against what rounding alone does), a little wider together."""
+
+from __future__ import annotations
+
+import json
+import random
+from pathlib import Path
+
+import pytest
+import torch
+
+import mini_llm_runtime_amd.models  # noqa: F401
+import schedules
+from helpers import make_runner, random_tokens
+from mini_llm_runtime_amd.weights import save_state_dict
+from test_pepulix import FAMILIES, _attn, _compare, _dense, _latent, _memory, _model, _moe, _ops, _rot, make_weights
+
+
+def _draw_rot(rng: random.Random, most: int, scaled: bool) -> dict:
+    dims = rng.choice([d for d in (2, 4, 8, 16, 32, 64, most) if d <= most and d % 2 == 0])
+    scaling = None
+    if scaled and rng.random() < 0.6:
+        scaling = (rng.choice([2.0, 4.0, 8.0, 32.0]), rng.choice([16, 64, 256, 4096]), rng.choice([4.0, 8.0, 32.0]), rng.choice([0.5, 1.0, 2.0]))
+    return _rot(rng.choice([100.0, 10000.0, 500000.0]), dims, scaling)
+
+
+def draw_config(seed: int) -> dict:
+    rng = random.Random(seed)
+    width = rng.choice([48, 64, 70, 72, 96, 100, 128, 160, 192, 256])
+    shared_values = (rng.choice([1, 2, 4]), rng.choice([8, 16, 24, 32, 64]))  # kv heads and width of mixed values
+    layers = []
+    for _ in range(rng.randint(1, 5)):
+        roll = rng.random()
+        if roll < 0.25:
+            mlp = None
+        elif roll < 0.6:
+            mlp = _dense(rng.choice([24, 40, 45, 64, 136, 320]))
+        else:
+            experts, identity = rng.choice([1, 2, 3, 5, 8, 16]), rng.choice([0, 0, 1, 2, 4])
+            mlp = _moe(rng.choice([8, 16, 24, 40, 50, 96]), experts, identity, rng.randint(1, min(4, experts + identity)))
+        kind = rng.choice(["attention", "latent", "memory"])
+        if kind == "attention":
+            v_mix = rng.random() < 0.6
+            kv = shared_values[0] if v_mix else rng.choice([1, 2, 3, 4])
+            heads = kv * rng.choice([1, 2, 3, 4])
+            dim = rng.choice([8, 16, 20, 32, 48, 64, 128])
+            vdim = shared_values[1] if v_mix else rng.choice([dim, 8, 12, 16, 32, 40, 64, 96])
+            rot = None if rng.random() < 0.2 else _draw_rot(rng, dim - dim % 2, scaled=False)
+            mixer = _attn(heads, kv, dim, vdim, round(rng.uniform(0.08, 0.4), 3), rot, v_mix)
+        elif kind == "latent":
+            heads = rng.choice([1, 2, 3, 4, 6, 8, 12])
+            dim = rng.choice([8, 10, 16, 24, 32, 64])
+            vdim = rng.choice([dim, 8, 12, 16, 32, 48])
+            rot_dim = rng.choice([2, 4, 6, 8, 16, 32, 64])
+            mixer = _latent(
+                heads, dim, rot_dim, vdim, rng.choice([8, 20, 24, 40, 64, 96, 128, 192]), rng.choice([4, 9, 16, 40, 80, 128]),
+                round(rng.uniform(0.08, 0.3), 3), _draw_rot(rng, rot_dim, scaled=True),
+            )
+        else:
+            heads = rng.choice([1, 2, 3, 4, 6, 8])
+            dim = rng.choice([4, 8, 16, 20, 32, 48, 64, 100, 128])
+            mixer = _memory(heads, dim, rng.choice([dim, 8, 12, 16, 32, 40, 64, 96]), rng.choice([5.0, 10.0, 15.0, 30.0]))
+        layers.append((mixer, mlp))
+    streams = rng.choice([None, 1, 2, 3, 4, 4, 6])
+    return _model(rng.randint(50, 600), width, rng.choice([1e-5, 1e-6]), layers, streams, rng.choice([None, 8.0, 15.0, 30.0]))
+
+
+def _run(tmp_path, seed: int, backend: str, dtype: torch.dtype) -> None:
+    cfg = draw_config(seed)
+    rng = random.Random(1000 + seed)
+    folder = Path(tmp_path) / f"drawn{seed}"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(cfg))
+    weights = make_weights(cfg, seed)
+    save_state_dict(folder / "model.safetensors", weights)
+    longest = 200 if backend == "hip" else 40
+    requests = {f"r{i}": random_tokens(rng.randint(1, longest), cfg["vocab"], seed * 10 + i) for i in range(rng.randint(2, 4))}
+    family = rng.choice(sorted(FAMILIES))
+    steps = FAMILIES[family](requests)
+    bs = rng.choice([4, 8, 16, 32])
+    _, _, cache, runner = make_runner(
+        folder, _ops(backend, dtype), block_size=bs, num_blocks=max(1, schedules.pages_needed(steps, bs)),
+        max_requests=schedules.most_live(steps),
+    )
+    cache.poison()
+    for bank in cache.state_banks.values():
+        bank.tensor.fill_(float("nan"))
+    got = schedules.run_schedule(runner, cache, steps)
+    try:
+        _compare(got, requests, weights, cfg, dtype, f32_bound=1e-3, together=4e-2)
+    except AssertionError as e:
+        raise AssertionError(f"{e}\nconfiguration {seed}: {json.dumps(cfg)}; {family}, pages of {bs}") from None
+    cache.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_drawn_configuration_on_the_stand_in(tmp_path, seed):
+    _run(tmp_path, seed, "double", torch.float32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(32))
+def test_drawn_configuration(tmp_path, seed):
+    _run(tmp_path, seed, "hip", torch.float32 if seed % 2 else torch.bfloat16)
