@@ -2,8 +2,8 @@
 mechanism.  It shares no code with the engine and exists to be compared with it.
 
 `config` is the decoder's config.json as a dict, `weights` a dict of float64 tensors under the
-checkpoint's own names.  `rounded(weights)` and the `round_to` argument of `forward` make the yardstick for
-ill-conditioned rows: the same arithmetic with every product's inputs rounded to bfloat16.
+checkpoint's own names.  The `round_to` argument of `forward` makes the yardstick for ill-conditioned rows:
+the same arithmetic with every product's inputs rounded to bfloat16.
 """
 
 from __future__ import annotations
@@ -27,10 +27,6 @@ def unit_rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return unit_rms(x, eps) * weight
-
-
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z**3)))
 
 
 def silu(z: torch.Tensor) -> torch.Tensor:
@@ -173,12 +169,17 @@ def dense_ff(w, p: str, h: torch.Tensor, round_to=None) -> torch.Tensor:
     return _r(inner, round_to) @ w[p + "down"].T + w[p + "down.b"]
 
 
-def route(w, p: str, mlp: Mapping, h: torch.Tensor):
-    """ids [T, top] and weights [T, top] of the chosen experts."""
+def route(w, p: str, mlp: Mapping, h: torch.Tensor, notes: Optional[dict] = None):
+    """ids [T, top] and weights [T, top] of the chosen experts.  `notes["margins"]` receives, per token, by how
+    much the last chosen expert's choice score leads the first one left out (a close call is a coin flip once
+    anything is rounded)."""
     top = int(mlp["router"]["top"])
     s = torch.softmax(h @ w[p + "router"].T, -1)
     choice = s + w[p + "correction"]
     ids = torch.topk(choice, top, dim=-1).indices
+    if notes is not None and choice.shape[-1] > top:
+        ranked = choice.sort(-1, descending=True).values
+        notes.setdefault("margins", []).append(ranked[:, top - 1] - ranked[:, top])
     chosen = torch.gather(s, 1, ids)
     return ids, chosen / (chosen.sum(-1, keepdim=True) + 1e-20)
 
@@ -188,10 +189,10 @@ def expert_ff(w, p: str, h: torch.Tensor, round_to=None) -> torch.Tensor:
     return _r(inner, round_to) @ w[p + "down"].T
 
 
-def moe_ff(w, p: str, mlp: Mapping, h: torch.Tensor, round_to=None) -> torch.Tensor:
+def moe_ff(w, p: str, mlp: Mapping, h: torch.Tensor, round_to=None, notes: Optional[dict] = None) -> torch.Tensor:
     real = int(mlp["router"]["experts"])
     hr = _r(h, round_to)
-    ids, weights = route(w, p, mlp, hr)
+    ids, weights = route(w, p, mlp, hr, notes)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, a in zip(ids[t].tolist(), weights[t]):
@@ -199,14 +200,18 @@ def moe_ff(w, p: str, mlp: Mapping, h: torch.Tensor, round_to=None) -> torch.Ten
     return out
 
 
-def feed_forward(w, p: str, mlp: Mapping, h: torch.Tensor, round_to=None) -> torch.Tensor:
-    return dense_ff(w, p, h, round_to) if mlp["kind"] == "dense" else moe_ff(w, p, mlp, h, round_to)
+def feed_forward(w, p: str, mlp: Mapping, h: torch.Tensor, round_to=None, notes: Optional[dict] = None) -> torch.Tensor:
+    return dense_ff(w, p, h, round_to) if mlp["kind"] == "dense" else moe_ff(w, p, mlp, h, round_to, notes)
 
 
 # ---- the model ------------------------------------------------------------------------------------------
 
-def forward(config: Mapping, weights: Mapping[str, torch.Tensor], tokens, round_to: Optional[torch.dtype] = None):
-    """logits [T, vocab] and the stream after every layer [layers, T, width] (the sum of the streams)."""
+def forward(
+    config: Mapping, weights: Mapping[str, torch.Tensor], tokens, round_to: Optional[torch.dtype] = None,
+    notes: Optional[dict] = None,
+):
+    """logits [T, vocab] and the stream after every layer [layers, T, width] (the sum of the streams).  `notes`
+    (a dict) receives what a comparison may want to know besides (see `route`)."""
     w = weights
     eps = float(config["norm"]["eps"])
     x0 = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
@@ -225,7 +230,7 @@ def forward(config: Mapping, weights: Mapping[str, torch.Tensor], tokens, round_
                 u = xs[0]
             h = rms_norm(u, w[f"{p}norm{q}"], eps)
             if q == 2:
-                y = feed_forward(w, p + "mlp.", what, h, round_to)
+                y = feed_forward(w, p + "mlp.", what, h, round_to, notes)
             elif what == "attention":
                 y = sigmoid_attention(w, p + "mix.", layer["mixer"], h, eps, shared, round_to)
             elif what == "latent_attention":

@@ -238,6 +238,9 @@ GPU_CASES = [
 ]
 
 
+CLOSE_CALL = 3e-3  # of a router's choice scores, which are probabilities plus a correction
+
+
 def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2, together=3e-2):
     """float32: every value within 1e-4 of the logits' size.  bfloat16: all rows together within 3 % (relative
     L2, the mean over the vocabulary taken off); every row within 6 %, but for a few (one in twenty, and as many
@@ -245,13 +248,20 @@ def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2,
     of their request (the plain implementation with the inputs of its products rounded to bfloat16): where a
     router's two candidates are nearly tied, or a memory's denominator is near its floor, rounding moves a row
     by percents in the plain implementation as in the engine.  A wrong key, page, slot, state or expert changes
-    most rows, by half and more."""
+    most rows, by half and more.  Rows at which a router's choice is a close call in the plain implementation
+    (the last chosen expert leads the first one left out by less than `CLOSE_CALL`) are left out in bfloat16:
+    there the engine's own roundings may send the token to the other expert while the rounded plain implementation
+    happens not to, and the two experts' weights can differ by a quarter of the row."""
     assert got, "no logits came back"
     w64 = _f64(weights)
     num = den = 0.0
     loose = rows = loose_alone = 0
     for rid, toks in requests.items():
-        ref, _ = plain.forward(cfg, w64, toks)
+        notes: dict = {}
+        ref, _ = plain.forward(cfg, w64, toks, notes=notes)
+        close = torch.zeros(len(toks), dtype=torch.bool)
+        for margin in notes.get("margins", []):
+            close |= margin.abs() < CLOSE_CALL
         ref = ref - ref.mean(-1, keepdim=True)
         size = float(ref.pow(2).mean().sqrt())
         if dtype != torch.float32:
@@ -268,6 +278,8 @@ def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2,
                 continue
             rows += 1
             rel = float(diff.pow(2).sum().sqrt() / ref[pos].pow(2).sum().sqrt())
+            if rel >= row_bound and bool(close[pos]):
+                continue
             if rel >= row_bound:
                 loose += 1
                 assert rel < 4.0 * max(float(alone.max()), row_bound / 2), f"{rid}:{pos}: relative error {rel:.3e}, rounding alone up to {float(alone.max()):.3e}"
