@@ -268,9 +268,10 @@ __global__ __launch_bounds__(256) void head_norm_rope_write_kernel(
 //   C' = exp(f + m - m') C + exp(i - m') k v^T,  n' likewise with k alone,
 //   o = C'^T q / (max(|n' . q|, exp(-m')) + 1e-6),  q scaled by q_scale.
 // An entry that starts its request starts from zeros (m = 0 too) whatever its row holds.  A workgroup of four
-// wavefronts owns 64 value columns of one head of one entry: lane (g, c) of a wavefront holds rows g, g + 4, ... of
-// column c of C and the same rows of n; eight tokens' q and k at a time go through LDS, rows beyond dim as zeros,
-// so the inner loops have no conditions.
+// wavefronts owns 64 value columns of one head of one entry: lane (g, c) of a wavefront holds a quarter of the rows
+// of column c of C (consecutive ones: 16-byte LDS reads) and the same rows of n; eight tokens' q and k at a time go
+// through LDS, rows beyond dim as zeros, so the inner loops have no conditions, and the eight after them are on
+// their way from memory meanwhile.
 constexpr int kMemTokens = 8;
 constexpr int kMemRun = 64;  // tokens of a run when long entries are walked in runs
 
@@ -309,15 +310,16 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ q_starts, float cap, float q_scale, float* __restrict__ out,
     int heads, int dim, int vdim, int entries, float* __restrict__ runs, float* __restrict__ run_gates) {
   constexpr int MAXD = 4 * R;
-  __shared__ __attribute__((aligned(16))) float sq[kMemTokens][MAXD];
-  __shared__ __attribute__((aligned(16))) float sk[kMemTokens][MAXD];
+  constexpr int kGroup = R + 4;  // floats of a group of rows in LDS: the four groups' 16-byte reads fall into banks of their own
+  __shared__ __attribute__((aligned(16))) float sq[kMemTokens][4][kGroup];
+  __shared__ __attribute__((aligned(16))) float sk[kMemTokens][4][kGroup];
   __shared__ float sv[kMemTokens][64];
   __shared__ float sg[kMemTokens][2];
   const int h = blockIdx.y;
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int wave = tid / kWave;
-  const int g = lane / 16;
+  const int g = lane / 16;  // this lane's rows: g * R .. g * R + R - 1
   const int c_local = wave * 16 + lane % 16;
   const int col = blockIdx.z * 64 + c_local;
   const bool col_ok = col < vdim;
@@ -338,38 +340,82 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
     src = dst = runs + (static_cast<int64_t>(blockIdx.x) * heads + h) * per_head;
   }
 
-  float C[R], n[R];
+  // The next eight tokens' q, k, v and gate sums are asked for while the present eight are walked, and wait in
+  // registers: a thread carries kPer numbers of q and of k, two of v and (the first eight threads) a token's gates.
+  constexpr int kPer = kMemTokens * MAXD / 256;
+  float rq[kPer], rk[kPer], rv[2], rgate[2];
+  auto fetch = [&](int t0) {
+    const int nb = min(kMemTokens, t_end - t0);
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      const int idx = tid + u * 256;
+      const int tt = idx / MAXD;
+      const int r = idx - tt * MAXD;
+      const bool in = tt < nb && r < dim;
+      const float* row = p + static_cast<int64_t>(t0 + (in ? tt : 0)) * width + h * dim + (in ? r : 0);
+      rq[u] = in ? row[q_off] * q_scale : 0.f;
+      rk[u] = in ? row[k_off] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int idx = tid + u * 256;
+      const int tt = idx / 64;
+      const int c = blockIdx.z * 64 + (idx - tt * 64);
+      const bool in = tt < nb && c < vdim;
+      rv[u] = in ? p[static_cast<int64_t>(t0 + tt) * width + v_off + h * vdim + c] : 0.f;
+    }
+    rgate[0] = rgate[1] = 0.f;
+    if (tid < nb) {
+      const float* row = p + static_cast<int64_t>(t0 + tid) * width;
+      rgate[0] = row[i_off + h];
+      rgate[1] = row[f_off + h];
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+      const int idx = tid + u * 256;
+      const int tt = idx / MAXD;
+      const int r = idx - tt * MAXD;
+      sq[tt][r / R][r % R] = rq[u];
+      sk[tt][r / R][r % R] = rk[u];
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int idx = tid + u * 256;
+      sv[idx / 64][idx % 64] = rv[u];
+    }
+    if (tid < kMemTokens) {
+      sg[tid][0] = cap * tanhf(rgate[0] / cap);
+      sg[tid][1] = log_sigmoid(cap * tanhf(rgate[1] / cap));
+    }
+  };
+  fetch(t_begin);
+
+  // n is the same for every column: a wavefront's 64 lanes share its rows among them (lane (g, c) holds rows
+  // g * R + c * NR .. + NR - 1) and n . q is a sum over the wavefront
+  constexpr int NR = R / 16;
+  const int n_at = (lane % 16) * NR;  // within the lane's group of rows
+  float C[R], n[NR];
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    const int r = g + 4 * j;
-    const bool in = r < dim && !fresh;
-    C[j] = (in && col_ok) ? src[static_cast<int64_t>(r) * vdim + col] : 0.f;
-    n[j] = in ? src[static_cast<int64_t>(dim) * vdim + r] : 0.f;
+    const int r = g * R + j;
+    C[j] = (r < dim && !fresh && col_ok) ? src[static_cast<int64_t>(r) * vdim + col] : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < NR; ++u) {
+    const int r = g * R + n_at + u;
+    n[u] = (r < dim && !fresh) ? src[static_cast<int64_t>(dim) * vdim + r] : 0.f;
   }
   float m = fresh ? (MODE == kRunSums ? -INFINITY : 0.f) : src[static_cast<int64_t>(dim) * vdim + dim];
   float f_sum = 0.f;
 
   for (int t0 = t_begin; t0 < t_end; t0 += kMemTokens) {
     const int nb = min(kMemTokens, t_end - t0);
+    __syncthreads();  // the tokens before are walked
+    stash();
     __syncthreads();
-    for (int idx = tid; idx < nb * MAXD; idx += 256) {
-      const int tt = idx / MAXD;
-      const int r = idx - tt * MAXD;
-      const float* row = p + static_cast<int64_t>(t0 + tt) * width;
-      sq[tt][r] = r < dim ? row[q_off + h * dim + r] * q_scale : 0.f;
-      sk[tt][r] = r < dim ? row[k_off + h * dim + r] : 0.f;
-    }
-    for (int idx = tid; idx < nb * 64; idx += 256) {
-      const int tt = idx / 64;
-      const int c = blockIdx.z * 64 + (idx - tt * 64);
-      sv[tt][idx - tt * 64] = c < vdim ? p[static_cast<int64_t>(t0 + tt) * width + v_off + h * vdim + c] : 0.f;
-    }
-    if (tid < nb) {
-      const float* row = p + static_cast<int64_t>(t0 + tid) * width;
-      sg[tid][0] = cap * tanhf(row[i_off + h] / cap);
-      sg[tid][1] = log_sigmoid(cap * tanhf(row[f_off + h] / cap));
-    }
-    __syncthreads();
+    if (t0 + kMemTokens < t_end) fetch(t0 + kMemTokens);  // on their way during the walk
     for (int tt = 0; tt < nb; ++tt) {
       const float ig = sg[tt][0];
       const float fg = sg[tt][1];
@@ -381,21 +427,24 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
       const float v = sv[tt][c_local] * take;
       float num = 0.f, nq = 0.f;
 #pragma unroll
-      for (int j = 0; j < R; ++j) {
-        const float kv = sk[tt][g + 4 * j];
-        const float qv = sq[tt][g + 4 * j];
-        C[j] = fmaf(keep, C[j], kv * v);
-        n[j] = fmaf(keep, n[j], kv * take);
-        if constexpr (MODE != kRunSums) {
-          num = fmaf(C[j], qv, num);
-          nq = fmaf(n[j], qv, nq);
+      for (int u = 0; u < NR; ++u) {
+        n[u] = fmaf(keep, n[u], sk[tt][g][n_at + u] * take);
+        nq = fmaf(n[u], sq[tt][g][n_at + u], nq);
+      }
+#pragma unroll
+      for (int j = 0; j < R; j += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(&sk[tt][g][j]);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(&sq[tt][g][j]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          C[j + e] = fmaf(keep, C[j + e], k4[e] * v);
+          if constexpr (MODE != kRunSums) num = fmaf(C[j + e], q4[e], num);
         }
       }
       if constexpr (MODE != kRunSums) {
         num += __shfl_xor(num, 16, kWave);
         num += __shfl_xor(num, 32, kWave);
-        nq += __shfl_xor(nq, 16, kWave);
-        nq += __shfl_xor(nq, 32, kWave);
+        nq = wave_sum(nq);
         if (g == 0 && col_ok)
           out[(static_cast<int64_t>(t0 + tt) * heads + h) * vdim + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
       }
@@ -410,10 +459,14 @@ __global__ __launch_bounds__(256) void matrix_memory_scan_kernel(
   }
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    const int r = g + 4 * j;
-    if (r < dim) {
-      if (col_ok) dst[static_cast<int64_t>(r) * vdim + col] = C[j];
-      if (blockIdx.z == 0 && wave == 0 && lane % 16 == 0) dst[static_cast<int64_t>(dim) * vdim + r] = n[j];
+    const int r = g * R + j;
+    if (r < dim && col_ok) dst[static_cast<int64_t>(r) * vdim + col] = C[j];
+  }
+  if (blockIdx.z == 0 && wave == 0) {
+#pragma unroll
+    for (int u = 0; u < NR; ++u) {
+      const int r = g * R + n_at + u;
+      if (r < dim) dst[static_cast<int64_t>(dim) * vdim + r] = n[u];
     }
   }
   if (MODE == kWholeEntries && blockIdx.z == 0 && tid == 0) dst[static_cast<int64_t>(dim) * vdim + dim] = m;
