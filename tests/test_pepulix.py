@@ -238,7 +238,7 @@ GPU_CASES = [
 ]
 
 
-CLOSE_CALL = 3e-3  # of a router's choice scores, which are probabilities plus a correction
+CLOSE_CALL = 2.5e-2  # of a router's choice scores (probabilities plus a correction): what the bfloat16 stream's error of a percent or two moves them by
 
 
 def _compare(got, requests, weights, cfg, dtype, f32_bound=1e-4, row_bound=6e-2, together=3e-2):
