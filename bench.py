@@ -47,6 +47,9 @@ the Qwen2 decoder of the same width, heads, head size, feed-forward width, layer
 The points named `side-*` (`VOBISUN_POINTS`; not among the default points either) run the Vobisun decoder
 (parallel layers whose mixer is windowed attention with pooled blocks beside linear attention with a decay
 per key channel, a short convolution before the mixer, a looped span of layers) beside that same Qwen2 twin.
+The points named `streams-*` (`PEPULIX_POINTS`; not among the default points) run the Pepulix decoder (four residual
+streams; layers of latent attention with a query latent, matrix memories and attention with sigmoid weights in turn;
+dense feed-forwards with biases and a mixture of gated experts) beside that Qwen2 twin.
 `reference`: the reference's own published measurements, run here at their parameters with the
 0.5B shape (random weights and token ids of the published lengths; its figures are of an RTX 3060
 laptop GPU in float16 and stand beside for scale): the burst of 8 short requests under continuous and

@@ -206,8 +206,9 @@ int mlr_retention_scan(float* projected, int width, float* state, int state_rows
                        int heads, int dim, int vdim, int chunked, int total_tokens, float* scratch, int64_t scratch_floats,
                        hipStream_t stream);
 
-// out[t * out_row + h * vdim + :] = retained[t, h, :] / rms(retained[t, h, :]) * norm_weight * silu(projected[t,
-// gate_offset + h * vdim + :]) * out_scale; norm_weight [vdim] is shared by the heads (null: none).
+// out[t * out_row + h * vdim + :] = retained[t, h, :] / rms(retained[t, h, :]) * norm_weight * act(projected[t,
+// gate_offset + h * vdim + :]) * out_scale; norm_weight [vdim] is shared by the heads, or with `weight_per_head`
+// [heads * vdim] (null: none); act is silu (gate_kind 0) or the sigmoid (1).
 int mlr_retention_gate(const float* retained, const float* projected, int width, int gate_offset, void* out, int dtype,
                        int tokens, int heads, int vdim, float eps, const void* norm_weight, int weight_is_f32,
                        float out_scale, int64_t out_row, int weight_per_head, int gate_kind, hipStream_t stream);
@@ -305,10 +306,11 @@ int mlr_sample_static(const float* logits, const float* temperature, const float
                       int rows, int vocab, hipStream_t stream);
 
 // Routed experts (moe.hip).  mlr_moe_route: per token, from the router's float32 logits [tokens,
-// experts]: s = sigmoid(z), choice scores c = s + correction (float32 [experts], or null); the
+// experts]: s = sigmoid(z) (score_kind 0) or softmax(z) over all experts (1), choice scores c = s + correction (float32 [experts], or null); the
 // expert axis is cut into `groups` contiguous blocks of experts / groups; block score = top-2 sum of
 // c; eligible are the experts of the `keep` highest blocks; ids [tokens, top] = arg-top-`top` of c over
-// the eligible (ties to the lower index), weights [tokens, top] = s[id] * scale.
+// the eligible (ties to the lower index), weights [tokens, top] = s[id] * scale, with `normalise` divided by the
+// sum of a token's chosen s (+ 1e-20) first.
 int mlr_moe_route(const float* logits, const float* correction, int* ids, float* weights, int tokens, int experts,
                   int top, int groups, int keep, float scale, int score_kind, int normalise, hipStream_t stream);
 // out[j, t, :] = weights[t, j] * h[t, :] where ids[t, j] >= first: experts without matrices that hand their input on.
