@@ -655,6 +655,35 @@ def test_schedule_matches_plain(tmp_path, which, family, backend, dtype):
     assert all(g.allocator.free_count == g.num_blocks for g in cache.groups), "pages were not given back"
 
 
+@pytest.mark.parametrize("dtype", GPU_CASES)
+def test_long_decoding(tmp_path, dtype):
+    """Two hundred tokens decoded one by one behind a prompt (replayed steps, partitions of the keys that grow,
+    page after page taken, the memory's state swapped at every commit), two requests side by side."""
+    folder, cfg, weights = make_dir(tmp_path, "D")
+    requests = {"a": random_tokens(330, cfg["vocab"], 21), "b": random_tokens(263, cfg["vocab"], 22)}
+    steps = []
+    for pos in range(330):  # a's prompt of 130 and b's of 63 in one step each, then a token of each per step
+        entries = []
+        for rid, toks in requests.items():
+            head = len(toks) - 200
+            if pos == head - 1:
+                entries.append({"id": rid, "tokens": toks[:head], "want": list(range(head))})
+            elif head <= pos < len(toks):
+                entries.append({"id": rid, "tokens": [toks[pos]], "want": [0]})
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": []})
+    steps[-1]["end"] = ["a"]
+    for step in reversed(steps):
+        if any(e["id"] == "b" for e in step["entries"]):
+            step["end"] = step["end"] + ["b"]
+            break
+    _, _, cache, runner = make_runner(
+        folder, _ops("hip", dtype), block_size=16, num_blocks=schedules.pages_needed(steps, 16), max_requests=2
+    )
+    cache.poison()
+    _compare(schedules.run_schedule(runner, cache, steps), requests, weights, cfg, dtype)
+
+
 @pytest.mark.parametrize("backend,dtype", CASES)
 @pytest.mark.parametrize("which", ["A", "C"])
 def test_layer_outputs_match_plain(tmp_path, which, backend, dtype):
